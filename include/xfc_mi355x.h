@@ -1,0 +1,150 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of Renee's XFC layer step.
+ *
+ * Every entry point takes plain device pointers, sizes, leading dimensions (in
+ * elements) and an opaque stream (a hipStream_t cast to void*, NULL = default
+ * stream).  All work is enqueued on that stream; nothing here synchronises or
+ * allocates device memory.  Each returns XFC_OK (0) or one of the XFC_ERR_* codes;
+ * nothing ever terminates the process (the reference extension calls exit() on
+ * failure: xfc_gemm_kernel.cu:14-22, :102-103, :243-244).
+ *
+ * Number types: X, W, M (momentum) and G are IEEE half; products accumulate in
+ * fp32; dX, dW (when written) and split partial sums are fp32.
+ *
+ * "reference" below is microsoft/renee; file:line cites its sources.
+ */
+#ifndef XFC_MI355X_H
+#define XFC_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XFC_ABI_VERSION 1
+
+enum {
+  XFC_OK = 0,
+  XFC_ERR_INVALID = 1,   /* null pointer, negative or > 2^31-1 dimension */
+  XFC_ERR_LAYOUT = 2,    /* stride pattern that selects no GEMM mode */
+  XFC_ERR_ALIGN = 3,     /* pointer or leading dimension not 16-byte aligned */
+  XFC_ERR_WORKSPACE = 4, /* workspace NULL or smaller than *_workspace_bytes() */
+  XFC_ERR_HIP = 5,       /* kernel launch failed */
+  XFC_ERR_SHAPE = 6      /* operand shapes disagree / leading dimension too small */
+};
+
+const char* xfc_strerror(int code);
+int xfc_abi_version(void);
+
+/*
+ * The six-argument fused GEMM of the reference extension:
+ *   xfc_gemm(mat_in1, mat_in2, mat_out, alpha, beta, apply_sigmoid)   xfc_gemm.cpp:17-40
+ * with each 2-D tensor flattened to (pointer, rows, cols, stride0, stride1).
+ * M, N come from mat_out and K from mat_in2's rows (xfc_gemm_kernel.cu:49-51);
+ * the mode is chosen from the strides of the views passed in, as there:
+ *   apply_sigmoid, in1 row-major, in2 column-major:
+ *        out(fp16) = sigmoid(alpha*in1.in2 + beta*out)      xfc_gemm_kernel.cu:59-100
+ *   in1 column-major, in2 row-major:
+ *        out(fp32) = alpha*in1.in2 + beta*out               xfc_gemm_kernel.cu:113-150
+ *   in1 row-major, in2 row-major (contraction over the long axis, split):
+ *        out(fp32) = alpha*in1.in2 + beta*out               xfc_gemm_kernel.cu:151-241
+ * in1 and in2 are fp16.  With beta == 0 the old contents of out are never read.
+ * Operands whose leading dimensions are not multiples of 8 elements take a slow
+ * any-stride kernel instead of failing.  The row x row mode needs a workspace of
+ * xfc_gemm_workspace_bytes(M, N, K) bytes (the reference allocates and frees its
+ * split-K workspace inside the call, xfc_gemm_kernel.cu:224-227).
+ */
+size_t xfc_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int xfc_gemm(const void* in1, int64_t in1_rows, int64_t in1_cols, int64_t in1_s0, int64_t in1_s1,
+             const void* in2, int64_t in2_rows, int64_t in2_cols, int64_t in2_s0, int64_t in2_s1,
+             void* out, int64_t out_rows, int64_t out_cols, int64_t out_s0, int64_t out_s1,
+             float alpha, float beta, int apply_sigmoid,
+             void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Logits only: out[B x L] (fp16) = X[B x d] . W[L x d]^T.
+ * Replaces BCELossMultiNode.xfc_forward, dl_base.py:568-573 (torch.matmul(out=)).
+ */
+int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out, int64_t ldo,
+               int64_t B, int64_t L, int64_t d, void* stream);
+
+/*
+ * Forward + loss gradient in one pass, the loss itself never formed:
+ *   G[b][l] = fp16( sigmoid(sum_k X[b][k]*W[l][k]) - [l in positives(b)] )
+ * Replaces dl_base.py:591-594 (fused-sigmoid GEMM, then out[pos_x,pos_y] -= 1.0).
+ * A (row, label) pair listed more than once lowers G by 1 once, as the
+ * reference's non-accumulating indexed update does; pairs outside [0,B)x[0,L)
+ * are ignored.  Positives come either as CSR (rowptr int32[B+1], colidx
+ * int32[nnz]) or as the reference's COO pair (pos_x, pos_y int64[nnz],
+ * dl_base.py:934-936), in any order.
+ * G has leading dimension ldg >= L; when ldg >= round_up(L, 8) the columns
+ * L .. round_up(L,8)-1 are written as zero (xfc_dx / xfc_dw_update rely on it).
+ * Workspace: xfc_fwd_grad_workspace_bytes(L, nnz) bytes.
+ */
+size_t xfc_fwd_grad_workspace_bytes(int64_t L, int64_t nnz);
+int xfc_fwd_grad_csr(const void* X, int64_t ldx, const void* W, int64_t ldw,
+                     const int32_t* rowptr, const int32_t* colidx,
+                     void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, int64_t nnz,
+                     void* workspace, size_t workspace_bytes, void* stream);
+int xfc_fwd_grad_coo(const void* X, int64_t ldx, const void* W, int64_t ldw,
+                     const int64_t* pos_x, const int64_t* pos_y, int64_t nnz,
+                     void* G, int64_t ldg, int64_t B, int64_t L, int64_t d,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * dX[B x d] (fp32) = scale * G[B x L] . W[L x d].
+ * Replaces dl_base.py:602-608 (torch.addmm with alpha = loss scale; the dead
+ * split-K call at :604).  Needs ldg >= round_up(L,8) with zeroed pad columns
+ * (xfc_fwd_grad_* writes them) and xfc_dx_workspace_bytes(B, L, d) of workspace.
+ */
+size_t xfc_dx_workspace_bytes(int64_t B, int64_t L, int64_t d);
+int xfc_dx(const void* G, int64_t ldg, const void* W, int64_t ldw, float* dX, int64_t lddx,
+           int64_t B, int64_t L, int64_t d, float scale,
+           void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * dW = G^T . X, consumed tile by tile by the SGD-momentum update so that W and M
+ * make one round trip through memory:
+ *   g = dW + weight_decay*W ;  M = momentum*M + g ;  W = W - lr*M
+ * (fp32 arithmetic, W and M rounded to fp16 once on store).  Replaces
+ * dl_base.py:620-634 (dW GEMM) + dl_base.py:343 (apex FusedSGD.step, parameters
+ * main.py:178-179: dampening 0, no Nesterov, decay before momentum).  M must be
+ * zero before the first step.  If dW_out is non-NULL the fp32 dW is also written
+ * there (leading dimension ld_dw), for checking.
+ */
+int xfc_dw_update(const void* G, int64_t ldg, const void* X, int64_t ldx,
+                  void* W, int64_t ldw, void* M, int64_t ldm,
+                  int64_t B, int64_t L, int64_t d,
+                  float lr, float momentum, float weight_decay,
+                  float* dW_out, int64_t ld_dw, void* stream);
+
+/*
+ * Split gradient accumulation (dl_base.py:318-340, :623-633):
+ *   grad[L x d] (fp32) = G^T . X + beta*grad      beta = 0 first micro-batch, 1 after
+ * followed once per step by xfc_sgd_momentum over count = L*d contiguous elements.
+ */
+int xfc_dw(const void* G, int64_t ldg, const void* X, int64_t ldx, float* grad, int64_t ld_grad,
+           int64_t B, int64_t L, int64_t d, float beta, void* stream);
+int xfc_sgd_momentum(void* W, void* M, const float* grad, int64_t count,
+                     float lr, float momentum, float weight_decay, void* stream);
+
+/*
+ * One whole step for one batch (dl_base.py:303-344 with accum == 1):
+ * xfc_fwd_grad_csr, xfc_dx (with W before the update), xfc_dw_update.
+ * G is caller-provided scratch of B x ldg halves, ldg >= round_up(L,8)
+ * (the reference's preallocated `outsoft`, dl_base.py:176).
+ */
+size_t xfc_step_workspace_bytes(int64_t B, int64_t L, int64_t d, int64_t nnz);
+int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* M, int64_t ldm,
+                 const int32_t* rowptr, const int32_t* colidx, int64_t nnz,
+                 void* G, int64_t ldg, float* dX, int64_t lddx,
+                 int64_t B, int64_t L, int64_t d,
+                 float lr, float momentum, float weight_decay, float scale,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XFC_MI355X_H */

@@ -1,0 +1,762 @@
+// XFC layer step kernels for gfx950 and their C-ABI entry points.
+//
+//   fwd   : G = fp16( sigmoid(X . W^T) - Y )      Y from per-label-tile positive buckets
+//   dx    : dX = scale * G . W                    split over labels, fp32 partials + reduce
+//   dw    : dW = G^T . X, consumed in the tile by  M = mu*M + dW + wd*W ; W -= lr*M
+// plus the plain six-argument GEMM the reference extension exposes.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/xfc_mi355x.h"
+#include "gemm_core.hpp"
+
+namespace xfc {
+
+// ---------------------------------------------------------------------------------------------
+// helpers
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float sigmoidf_fast(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
+}
+
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Tiles that
+// share an operand slice are given ids that land on one XCD next to each other:
+// id -> (inner, outer) with `inner` (size n_inner) varying fastest among ids of one XCD.
+__device__ __forceinline__ void xcd_map(int id, int n_inner, int& inner, int& outer) {
+  const int xcd = id & 7, local = id >> 3;
+  inner = local % n_inner;
+  outer = (local / n_inner) * 8 + xcd;
+}
+
+// ---------------------------------------------------------------------------------------------
+// positives: bucket a sparse label list by label tile
+// ---------------------------------------------------------------------------------------------
+// One workgroup.  Input is CSR (rowptr/colidx, pos_x == nullptr) or COO (pos_x/pos_y int64).
+// Output: bucket_ptr[n_tiles+1] and (ent_row, ent_col)[nnz] grouped by col / tile_w.
+// Pairs whose row or column is out of range are dropped.  cursor[n_tiles] is scratch.
+__global__ void __launch_bounds__(1024) bucket_positives_kernel(
+    const int32_t* __restrict__ rowptr, const int32_t* __restrict__ colidx, const int64_t* __restrict__ pos_x,
+    const int64_t* __restrict__ pos_y, int64_t nnz, int B, int64_t L, int tile_w, int n_tiles,
+    int32_t* __restrict__ bucket_ptr, int32_t* __restrict__ cursor, int32_t* __restrict__ ent_row,
+    int32_t* __restrict__ ent_col) {
+  __shared__ int32_t part[1024];
+  const int t = threadIdx.x;
+  for (int i = t; i < n_tiles; i += 1024) cursor[i] = 0;
+  __syncthreads();
+  if (pos_x) {
+    for (int64_t p = t; p < nnz; p += 1024) {
+      const int64_t r = pos_x[p], c = pos_y[p];
+      if (r >= 0 && r < B && c >= 0 && c < L) atomicAdd(&cursor[(int)(c / tile_w)], 1);
+    }
+  } else {
+    for (int b = t; b < B; b += 1024)
+      for (int p = rowptr[b]; p < rowptr[b + 1]; ++p) {
+        const int64_t c = colidx[p];
+        if (c >= 0 && c < L) atomicAdd(&cursor[(int)(c / tile_w)], 1);
+      }
+  }
+  __syncthreads();
+  const int per = (n_tiles + 1023) / 1024;
+  const int lo = t * per, hi = min(n_tiles, lo + per);
+  int s = 0;
+  for (int i = lo; i < hi; ++i) s += cursor[i];
+  part[t] = s;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    int v = t >= off ? part[t - off] : 0;
+    __syncthreads();
+    part[t] += v;
+    __syncthreads();
+  }
+  int run = part[t] - s;
+  for (int i = lo; i < hi; ++i) {
+    const int c = cursor[i];
+    bucket_ptr[i] = run;
+    cursor[i] = run;
+    run += c;
+  }
+  if (t == 1023) bucket_ptr[n_tiles] = part[1023];
+  __syncthreads();
+  if (pos_x) {
+    for (int64_t p = t; p < nnz; p += 1024) {
+      const int64_t r = pos_x[p], c = pos_y[p];
+      if (r >= 0 && r < B && c >= 0 && c < L) {
+        const int at = atomicAdd(&cursor[(int)(c / tile_w)], 1);
+        ent_row[at] = (int)r;
+        ent_col[at] = (int)c;
+      }
+    }
+  } else {
+    for (int b = t; b < B; b += 1024)
+      for (int p = rowptr[b]; p < rowptr[b + 1]; ++p) {
+        const int64_t c = colidx[p];
+        if (c >= 0 && c < L) {
+          const int at = atomicAdd(&cursor[(int)(c / tile_w)], 1);
+          ent_row[at] = b;
+          ent_col[at] = (int)c;
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward: out = epilogue(alpha * X . W^T + beta * out)
+// ---------------------------------------------------------------------------------------------
+enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2 };
+
+using FwdCore = GemmCore<256, 128, 64, 2, 2, true, true>;
+constexpr int FWD_LDS_BYTES = FwdCore::STAGE_HALVES * 2;
+
+struct FwdArgs {
+  const half_t* X; int64_t ldx;     // M x K, K-contiguous
+  const half_t* W; int64_t ldw;     // N x K, K-contiguous
+  half_t* out; int64_t ldo;         // M x n_store, row-major
+  int M, N, K, n_store;             // columns N <= c < n_store are written as zero
+  float alpha, beta;
+  const int32_t* bucket_ptr; const int32_t* ent_row; const int32_t* ent_col;
+  int tiles_m, tiles_n;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(256, 2) fwd_kernel(FwdArgs a) {
+  using C = FwdCore;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  half_t* lds = reinterpret_cast<half_t*>(smem_raw);
+  int mt, nt;
+  xcd_map(blockIdx.x, a.tiles_m, mt, nt);
+  if (nt >= a.tiles_n) return;
+  const int m0 = mt * C::BM, n0 = nt * C::BN;
+  float16v acc[C::FM][C::FN];
+#pragma unroll
+  for (int i = 0; i < C::FM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  typename C::Operand oa{a.X, a.ldx, m0, a.M, a.K};
+  typename C::Operand ob{a.W, a.ldw, n0, a.N, a.K};
+  C::template run<1>(oa, ob, 0, a.K, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  // positives of this tile -> bitmap [label][row word]
+  uint32_t* bm = reinterpret_cast<uint32_t*>(smem_raw);
+  bool has = false;
+  if constexpr (MODE == FWD_GRAD) {
+    const int s = a.bucket_ptr[nt], e = a.bucket_ptr[nt + 1];
+    has = e > s;
+    if (has) {
+      for (int i = threadIdx.x; i < C::BN * (C::BM / 32); i += C::NT) bm[i] = 0u;
+      __syncthreads();
+      for (int p = s + threadIdx.x; p < e; p += C::NT) {
+        const int r = a.ent_row[p] - m0, c = a.ent_col[p] - n0;
+        if (r >= 0 && r < C::BM) atomicOr(&bm[c * (C::BM / 32) + (r >> 5)], 1u << (r & 31));
+      }
+      __syncthreads();
+    }
+  }
+#pragma unroll
+  for (int fm = 0; fm < C::FM; ++fm) {
+#pragma unroll
+    for (int fn = 0; fn < C::FN; ++fn) {
+      const int lcol = wn * C::TN + fn * 32 + (lane & 31);
+      const int col = n0 + lcol;
+      uint32_t word = 0u;
+      if constexpr (MODE == FWD_GRAD) {
+        if (has) word = bm[lcol * (C::BM / 32) + ((wm * C::TM + fm * 32) >> 5)];
+      }
+      if (col < a.n_store) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int lr = c_row(r, lane);
+          const int row = m0 + wm * C::TM + fm * 32 + lr;
+          if (row < a.M) {
+            half_t* dst = a.out + (int64_t)row * a.ldo + col;
+            float v = a.alpha * acc[fm][fn][r];
+            if (a.beta != 0.f) v += a.beta * (float)(*dst);
+            if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
+            if constexpr (MODE == FWD_GRAD) v -= (float)((word >> lr) & 1u);
+            if (col >= a.N) v = 0.f;
+            *dst = (half_t)v;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
+// ---------------------------------------------------------------------------------------------
+using DxCore = GemmCore<256, 128, 64, 2, 2, true, false>;
+constexpr int DX_LDS_BYTES = DxCore::STAGE_HALVES * 2;
+
+struct DxArgs {
+  const half_t* G; int64_t ldg;   // M x K, K-contiguous (K = labels)
+  const half_t* W; int64_t ldw;   // K x N, N-contiguous
+  float* part;                    // [splits][M][N]
+  int M, N, K;
+  int tiles_m, tiles_n, splits, k_per_split;  // k_per_split is a multiple of BK
+};
+
+__global__ void __launch_bounds__(256, 2) dx_kernel(DxArgs a) {
+  using C = DxCore;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  half_t* lds = reinterpret_cast<half_t*>(smem_raw);
+  int tile, split;
+  xcd_map(blockIdx.x, a.tiles_m * a.tiles_n, tile, split);
+  if (split >= a.splits) return;
+  const int mt = tile % a.tiles_m, nt = tile / a.tiles_m;
+  const int m0 = mt * C::BM, n0 = nt * C::BN;
+  float16v acc[C::FM][C::FN];
+#pragma unroll
+  for (int i = 0; i < C::FM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  const int64_t kb = (int64_t)split * a.k_per_split;
+  const int k_begin = (int)(kb < a.K ? kb : a.K);
+  const int k_end = (int)(kb + a.k_per_split < a.K ? kb + a.k_per_split : a.K);
+  typename C::Operand oa{a.G, a.ldg, m0, a.M, a.K};
+  typename C::Operand ob{a.W, a.ldw, n0, a.N, a.K};
+  C::template run<1>(oa, ob, k_begin, k_end, lds, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  float* part = a.part + (int64_t)split * a.M * a.N;
+#pragma unroll
+  for (int fm = 0; fm < C::FM; ++fm)
+#pragma unroll
+    for (int fn = 0; fn < C::FN; ++fn) {
+      const int col = n0 + wn * C::TN + fn * 32 + (lane & 31);
+      if (col < a.N) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
+          if (row < a.M) part[(int64_t)row * a.N + col] = acc[fm][fn][r];
+        }
+      }
+    }
+}
+
+// out[m][n] = alpha * sum_s part[s][m][n] + beta * out[m][n]; one thread per 4 columns.
+__global__ void __launch_bounds__(256) dx_reduce_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                        int64_t ldo, int M, int N, int splits, float alpha,
+                                                        float beta) {
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int nq = N / 4;
+  if (q >= (int64_t)M * nq) return;
+  const int m = (int)(q / nq), n = (int)(q % nq) * 4;
+  float4v s = {0.f, 0.f, 0.f, 0.f};
+  const float* p = part + (int64_t)m * N + n;
+  for (int i = 0; i < splits; ++i) s += *reinterpret_cast<const float4v*>(p + (int64_t)i * M * N);
+  float* o = out + (int64_t)m * ldo + n;
+  float4v r = alpha * s;
+  if (beta != 0.f) {
+    r[0] += beta * o[0]; r[1] += beta * o[1]; r[2] += beta * o[2]; r[3] += beta * o[3];
+  }
+  o[0] = r[0]; o[1] = r[1]; o[2] = r[2]; o[3] = r[3];
+}
+
+// ---------------------------------------------------------------------------------------------
+// dW = G^T . X; either written out (fp32, alpha/beta) or consumed by the momentum update
+// ---------------------------------------------------------------------------------------------
+enum DwMode { DW_OUT = 0, DW_UPDATE = 1 };
+
+using DwCore = GemmCore<128, 256, 64, 2, 2, false, false>;
+constexpr int DW_STAGE_PITCH = 72;  // floats per staged row (64 + 8: rows 4 apart land 32 banks apart)
+constexpr int DW_STAGE_BYTES = 4 * 32 * DW_STAGE_PITCH * 4;
+constexpr int DW_LDS_BYTES = DwCore::STAGE_HALVES * 2 > DW_STAGE_BYTES ? DwCore::STAGE_HALVES * 2 : DW_STAGE_BYTES;
+
+struct DwArgs {
+  const half_t* G; int64_t ldg;   // K x M (batch rows x labels), label-contiguous
+  const half_t* X; int64_t ldx;   // K x N, N-contiguous
+  int M, N, K;                    // labels, feature dims, batch rows
+  int g_cols;                     // readable columns of G per row (>= M, multiple of 8)
+  // DW_OUT
+  float* out; int64_t ldo; float alpha, beta;
+  // DW_UPDATE
+  half_t* Wt; int64_t ldw; half_t* Mo; int64_t ldm; float lr, mu, wd;
+  float* dw_dump; int64_t ld_dump;  // optional copy of dW (may be null)
+  int tiles_m, tiles_n;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
+  using C = DwCore;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  half_t* lds = reinterpret_cast<half_t*>(smem_raw);
+  int nt, mt;
+  xcd_map(blockIdx.x, a.tiles_n, nt, mt);
+  if (mt >= a.tiles_m) return;
+  const int m0 = mt * C::BM, n0 = nt * C::BN;
+  float16v acc[C::FM][C::FN];
+#pragma unroll
+  for (int i = 0; i < C::FM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  typename C::Operand oa{a.G, a.ldg, m0, a.g_cols, a.K};
+  typename C::Operand ob{a.X, a.ldx, n0, a.N, a.K};
+  C::template run<1>(oa, ob, 0, a.K, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  float* stage = reinterpret_cast<float*>(smem_raw) + wave * 32 * DW_STAGE_PITCH;
+#pragma unroll
+  for (int fm = 0; fm < C::FM; ++fm) {
+#pragma unroll
+    for (int fp = 0; fp < C::FN / 2; ++fp) {
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          stage[c_row(r, lane) * DW_STAGE_PITCH + 32 * q + (lane & 31)] = acc[fm][2 * fp + q][r];
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int cid = lane + 64 * i;
+        const int lr = cid >> 3, ch = cid & 7;
+        const int row = m0 + wm * C::TM + fm * 32 + lr;
+        const int col = n0 + wn * C::TN + fp * 64 + ch * 8;
+        if (row >= a.M || col >= a.N) continue;
+        const float4v v0 = *reinterpret_cast<const float4v*>(stage + lr * DW_STAGE_PITCH + ch * 8);
+        const float4v v1 = *reinterpret_cast<const float4v*>(stage + lr * DW_STAGE_PITCH + ch * 8 + 4);
+        float g[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        if constexpr (MODE == DW_OUT) {
+          float* o = a.out + (int64_t)row * a.ldo + col;
+          float4v o0, o1;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
+          if (a.beta != 0.f) {
+            o0 += a.beta * *reinterpret_cast<const float4v*>(o);
+            o1 += a.beta * *reinterpret_cast<const float4v*>(o + 4);
+          }
+          *reinterpret_cast<float4v*>(o) = o0;
+          *reinterpret_cast<float4v*>(o + 4) = o1;
+        } else {
+          half_t* wp = a.Wt + (int64_t)row * a.ldw + col;
+          half_t* mp = a.Mo + (int64_t)row * a.ldm + col;
+          half8 w = *reinterpret_cast<const half8*>(wp);
+          half8 m = *reinterpret_cast<const half8*>(mp);
+          if (a.dw_dump) {
+            float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
+            *reinterpret_cast<float4v*>(d) = v0;
+            *reinterpret_cast<float4v*>(d + 4) = v1;
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float wf = (float)w[e];
+            const float gg = g[e] + a.wd * wf;
+            const float mf = a.mu * (float)m[e] + gg;
+            m[e] = (half_t)mf;
+            w[e] = (half_t)(wf - a.lr * mf);
+          }
+          *reinterpret_cast<half8*>(mp) = m;
+          *reinterpret_cast<half8*>(wp) = w;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// any-stride fallback: one thread per output element
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) generic_gemm_kernel(const half_t* __restrict__ A, int64_t as0, int64_t as1,
+                                                           const half_t* __restrict__ Bm, int64_t bs0, int64_t bs1,
+                                                           void* out, int64_t os0, int64_t os1, int M, int N, int K,
+                                                           float alpha, float beta, int sigmoid, int out_half) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * N) return;
+  const int m = (int)(idx / N), n = (int)(idx % N);
+  float s = 0.f;
+  for (int k = 0; k < K; ++k) s += (float)A[m * as0 + k * as1] * (float)Bm[k * bs0 + n * bs1];
+  s *= alpha;
+  const int64_t o = m * os0 + n * os1;
+  if (out_half) {
+    half_t* p = reinterpret_cast<half_t*>(out) + o;
+    if (beta != 0.f) s += beta * (float)*p;
+    if (sigmoid) s = sigmoidf_fast(s);
+    *p = (half_t)s;
+  } else {
+    float* p = reinterpret_cast<float*>(out) + o;
+    if (beta != 0.f) s += beta * *p;
+    if (sigmoid) s = sigmoidf_fast(s);
+    *p = s;
+  }
+}
+
+// SGD-momentum on an fp32 gradient (used when dW was accumulated over micro-batches).
+__global__ void __launch_bounds__(256) sgd_momentum_kernel(half_t* __restrict__ W, half_t* __restrict__ Mo,
+                                                           const float* __restrict__ grad, int64_t n8, float lr,
+                                                           float mu, float wd) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  half8 w = reinterpret_cast<half8*>(W)[i];
+  half8 m = reinterpret_cast<half8*>(Mo)[i];
+  const float4v g0 = reinterpret_cast<const float4v*>(grad)[2 * i];
+  const float4v g1 = reinterpret_cast<const float4v*>(grad)[2 * i + 1];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float wf = (float)w[e];
+    const float gg = (e < 4 ? g0[e] : g1[e - 4]) + wd * wf;
+    const float mf = mu * (float)m[e] + gg;
+    m[e] = (half_t)mf;
+    w[e] = (half_t)(wf - lr * mf);
+  }
+  reinterpret_cast<half8*>(W)[i] = w;
+  reinterpret_cast<half8*>(Mo)[i] = m;
+}
+
+}  // namespace xfc
+
+// =============================================================================================
+// C ABI
+// =============================================================================================
+using namespace xfc;
+
+namespace {
+
+inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_launch() {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fprintf(stderr, "xfc: kernel launch failed: %s\n", hipGetErrorString(e));
+    return XFC_ERR_HIP;
+  }
+  return XFC_OK;
+}
+
+int num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
+    n = p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+  }
+  return n;
+}
+
+struct BucketWs {
+  int32_t *bucket_ptr, *cursor, *ent_row, *ent_col;
+};
+
+size_t bucket_ws_bytes(int64_t L, int64_t nnz) {
+  const int64_t n_tiles = round_up(ceil_div(L, FwdCore::BN), 8);
+  return (size_t)round_up((n_tiles + 1) * 4, 256) + (size_t)round_up(n_tiles * 4, 256) +
+         2 * (size_t)round_up((nnz > 0 ? nnz : 1) * 4, 256);
+}
+
+BucketWs carve_bucket_ws(void* ws, int64_t L, int64_t nnz) {
+  const int64_t n_tiles = round_up(ceil_div(L, FwdCore::BN), 8);
+  unsigned char* p = reinterpret_cast<unsigned char*>(ws);
+  BucketWs b;
+  b.bucket_ptr = reinterpret_cast<int32_t*>(p); p += round_up((n_tiles + 1) * 4, 256);
+  b.cursor = reinterpret_cast<int32_t*>(p); p += round_up(n_tiles * 4, 256);
+  b.ent_row = reinterpret_cast<int32_t*>(p); p += round_up((nnz > 0 ? nnz : 1) * 4, 256);
+  b.ent_col = reinterpret_cast<int32_t*>(p);
+  return b;
+}
+
+int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, half_t* out, int64_t ldo, int M,
+               int N, int K, int n_store, float alpha, float beta, const BucketWs* bk, hipStream_t st) {
+  FwdArgs a;
+  a.X = X; a.ldx = ldx; a.W = W; a.ldw = ldw; a.out = out; a.ldo = ldo;
+  a.M = M; a.N = N; a.K = K; a.n_store = n_store; a.alpha = alpha; a.beta = beta;
+  a.bucket_ptr = bk ? bk->bucket_ptr : nullptr;
+  a.ent_row = bk ? bk->ent_row : nullptr;
+  a.ent_col = bk ? bk->ent_col : nullptr;
+  a.tiles_m = ceil_div(M, FwdCore::BM);
+  a.tiles_n = ceil_div(n_store, FwdCore::BN);
+  const int64_t grid = (int64_t)a.tiles_m * round_up(a.tiles_n, 8);
+  if (grid <= 0) return XFC_OK;
+  if (grid > 0x7fffffff) return XFC_ERR_INVALID;
+  dim3 g((unsigned)grid), b(256);
+  if (mode == FWD_GRAD) hipLaunchKernelGGL(fwd_kernel<FWD_GRAD>, g, b, FWD_LDS_BYTES, st, a);
+  else if (mode == FWD_SIGMOID) hipLaunchKernelGGL(fwd_kernel<FWD_SIGMOID>, g, b, FWD_LDS_BYTES, st, a);
+  else hipLaunchKernelGGL(fwd_kernel<FWD_LINEAR>, g, b, FWD_LDS_BYTES, st, a);
+  return check_launch();
+}
+
+// Split count for dX: enough workgroups for two per CU, a multiple of 8 (one slice of the
+// label axis per XCD at a time), each slice a multiple of the k-step.
+void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& k_per_split) {
+  tiles_m = ceil_div(M, DxCore::BM);
+  tiles_n = ceil_div(N, DxCore::BN);
+  const int tiles = tiles_m * tiles_n;
+  int s = (2 * num_cus()) / (tiles > 0 ? tiles : 1);
+  s = s / 8 * 8;
+  if (s < 8) s = 8;
+  const int max_s = (int)round_up(ceil_div(K, DxCore::BK), 8);
+  if (s > max_s) s = max_s;
+  k_per_split = (int)round_up(ceil_div(K, s), DxCore::BK);
+  splits = s;
+}
+
+int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float* out, int64_t ldo, int M, int N, int K,
+              float alpha, float beta, void* ws, size_t ws_bytes, hipStream_t st) {
+  DxArgs a;
+  dx_plan(M, N, K, a.tiles_m, a.tiles_n, a.splits, a.k_per_split);
+  const size_t need = (size_t)a.splits * M * N * 4;
+  if (ws == nullptr || ws_bytes < need) return XFC_ERR_WORKSPACE;
+  a.G = G; a.ldg = ldg; a.W = W; a.ldw = ldw; a.part = reinterpret_cast<float*>(ws);
+  a.M = M; a.N = N; a.K = K;
+  const int64_t grid = (int64_t)a.tiles_m * a.tiles_n * a.splits;
+  if (grid <= 0 || M <= 0 || N <= 0) return XFC_OK;
+  hipLaunchKernelGGL(dx_kernel, dim3((unsigned)grid), dim3(256), DX_LDS_BYTES, st, a);
+  int rc = check_launch();
+  if (rc) return rc;
+  const int64_t nq = (int64_t)M * (N / 4);
+  hipLaunchKernelGGL(dx_reduce_kernel, dim3((unsigned)ceil_div(nq, 256)), dim3(256), 0, st, a.part, out, ldo, M, N,
+                     a.splits, alpha, beta);
+  return check_launch();
+}
+
+int launch_dw(int mode, DwArgs a, hipStream_t st) {
+  a.tiles_m = ceil_div(a.M, DwCore::BM);
+  a.tiles_n = ceil_div(a.N, DwCore::BN);
+  const int64_t grid = (int64_t)a.tiles_n * round_up(a.tiles_m, 8);
+  if (grid <= 0) return XFC_OK;
+  if (grid > 0x7fffffff) return XFC_ERR_INVALID;
+  if (mode == DW_UPDATE)
+    hipLaunchKernelGGL(dw_kernel<DW_UPDATE>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  else
+    hipLaunchKernelGGL(dw_kernel<DW_OUT>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  return check_launch();
+}
+
+int launch_generic(const void* in1, int64_t as0, int64_t as1, const void* in2, int64_t bs0, int64_t bs1, void* out,
+                   int64_t os0, int64_t os1, int M, int N, int K, float alpha, float beta, int sigmoid, int out_half,
+                   hipStream_t st) {
+  const int64_t total = (int64_t)M * N;
+  if (total <= 0) return XFC_OK;
+  hipLaunchKernelGGL(generic_gemm_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st,
+                     reinterpret_cast<const half_t*>(in1), as0, as1, reinterpret_cast<const half_t*>(in2), bs0, bs1,
+                     out, os0, os1, M, N, K, alpha, beta, sigmoid, out_half);
+  return check_launch();
+}
+
+bool dims_ok(int64_t v) { return v >= 0 && v <= 0x7fffffff; }
+
+}  // namespace
+
+extern "C" {
+
+const char* xfc_strerror(int code) {
+  switch (code) {
+    case XFC_OK: return "ok";
+    case XFC_ERR_INVALID: return "invalid argument (null pointer, negative or oversized dimension)";
+    case XFC_ERR_LAYOUT: return "unsupported operand layout: expected row x column (sigmoid), column x row, or row x row";
+    case XFC_ERR_ALIGN: return "operand pointer or leading dimension not aligned to 16 bytes";
+    case XFC_ERR_WORKSPACE: return "workspace missing or too small";
+    case XFC_ERR_HIP: return "HIP runtime error";
+    case XFC_ERR_SHAPE: return "operand shapes do not agree";
+    default: return "unknown error";
+  }
+}
+
+int xfc_abi_version(void) { return XFC_ABI_VERSION; }
+
+size_t xfc_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (!dims_ok(M) || !dims_ok(N) || !dims_ok(K)) return 0;
+  int tm, tn, s, kps;
+  dx_plan((int)M, (int)N, (int)K, tm, tn, s, kps);
+  return (size_t)s * M * N * 4;
+}
+
+int xfc_gemm(const void* in1, int64_t in1_rows, int64_t in1_cols, int64_t in1_s0, int64_t in1_s1, const void* in2,
+             int64_t in2_rows, int64_t in2_cols, int64_t in2_s0, int64_t in2_s1, void* out, int64_t out_rows,
+             int64_t out_cols, int64_t out_s0, int64_t out_s1, float alpha, float beta, int apply_sigmoid,
+             void* workspace, size_t workspace_bytes, void* stream) {
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int64_t M = out_rows, N = out_cols, K = in2_rows;
+  if (!dims_ok(M) || !dims_ok(N) || !dims_ok(K)) return XFC_ERR_INVALID;
+  if (in1_rows != M || in1_cols != K || in2_cols != N) return XFC_ERR_SHAPE;
+  if (M == 0 || N == 0) return XFC_OK;
+  if (!in1 || !in2 || !out) return XFC_ERR_INVALID;
+  const bool a_row = in1_s1 == 1, a_col = in1_s0 == 1, b_row = in2_s1 == 1, b_col = in2_s0 == 1;
+  if (apply_sigmoid) {
+    // out(fp16) = sigmoid(alpha * in1 . in2 + beta * out), in1 row-major, in2 column-major
+    if (!(a_row && b_col)) return XFC_ERR_LAYOUT;
+    const bool fast = out_s1 == 1 && in1_s0 % 8 == 0 && in2_s1 % 8 == 0 && K % 8 == 0 && aligned16(in1) &&
+                      aligned16(in2) && K > 0;
+    if (fast)
+      return launch_fwd(FWD_SIGMOID, (const half_t*)in1, in1_s0, (const half_t*)in2, in2_s1, (half_t*)out, out_s0,
+                        (int)M, (int)N, (int)K, (int)N, alpha, beta, nullptr, st);
+    return launch_generic(in1, in1_s0, in1_s1, in2, in2_s0, in2_s1, out, out_s0, out_s1, (int)M, (int)N, (int)K, alpha,
+                          beta, 1, 1, st);
+  }
+  if (a_col && b_row) {
+    // out(fp32) = alpha * in1 . in2 + beta * out, in1 column-major (G^T view), in2 row-major (X)
+    const bool fast = out_s1 == 1 && out_s0 % 4 == 0 && aligned16(out) && in1_s1 % 8 == 0 && in2_s0 % 8 == 0 &&
+                      N % 8 == 0 && M % 8 == 0 && aligned16(in1) && aligned16(in2) && K > 0;
+    if (fast) {
+      DwArgs a = {};
+      a.G = (const half_t*)in1; a.ldg = in1_s1; a.X = (const half_t*)in2; a.ldx = in2_s0;
+      a.M = (int)M; a.N = (int)N; a.K = (int)K; a.g_cols = (int)round_up(M, 8);
+      a.out = (float*)out; a.ldo = out_s0; a.alpha = alpha; a.beta = beta;
+      return launch_dw(DW_OUT, a, st);
+    }
+    return launch_generic(in1, in1_s0, in1_s1, in2, in2_s0, in2_s1, out, out_s0, out_s1, (int)M, (int)N, (int)K, alpha,
+                          beta, 0, 0, st);
+  }
+  if (a_row && b_row) {
+    // out(fp32) = alpha * in1 . in2 + beta * out, both row-major: contraction over in1's columns
+    const bool fast = out_s1 == 1 && in1_s0 % 8 == 0 && in2_s0 % 8 == 0 && N % 8 == 0 && K % 8 == 0 &&
+                      aligned16(in1) && aligned16(in2) && K > 0;
+    if (fast) {
+      return launch_dx((const half_t*)in1, in1_s0, (const half_t*)in2, in2_s0, (float*)out, out_s0, (int)M, (int)N,
+                       (int)K, alpha, beta, workspace, workspace_bytes, st);
+    }
+    return launch_generic(in1, in1_s0, in1_s1, in2, in2_s0, in2_s1, out, out_s0, out_s1, (int)M, (int)N, (int)K, alpha,
+                          beta, 0, 0, st);
+  }
+  return XFC_ERR_LAYOUT;
+}
+
+int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out, int64_t ldo, int64_t B, int64_t L,
+               int64_t d, void* stream) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
+  if (B == 0 || L == 0) return XFC_OK;
+  if (!X || !W || !out || d <= 0) return XFC_ERR_INVALID;
+  if (ldx % 8 || ldw % 8 || d % 8 || !aligned16(X) || !aligned16(W)) return XFC_ERR_ALIGN;
+  return launch_fwd(FWD_LINEAR, (const half_t*)X, ldx, (const half_t*)W, ldw, (half_t*)out, ldo, (int)B, (int)L, (int)d,
+                    (int)L, 1.0f, 0.0f, nullptr, reinterpret_cast<hipStream_t>(stream));
+}
+
+size_t xfc_fwd_grad_workspace_bytes(int64_t L, int64_t nnz) {
+  if (!dims_ok(L) || nnz < 0) return 0;
+  return bucket_ws_bytes(L, nnz);
+}
+
+static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw, const int32_t* rowptr,
+                         const int32_t* colidx, const int64_t* pos_x, const int64_t* pos_y, int64_t nnz, void* G,
+                         int64_t ldg, int64_t B, int64_t L, int64_t d, void* ws, size_t ws_bytes, hipStream_t st) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d) || nnz < 0 || nnz > 0x7fffffff) return XFC_ERR_INVALID;
+  if (B == 0 || L == 0) return XFC_OK;
+  if (!X || !W || !G || d <= 0) return XFC_ERR_INVALID;
+  if (nnz > 0 && !((rowptr && colidx) || (pos_x && pos_y))) return XFC_ERR_INVALID;
+  if (ldx % 8 || ldw % 8 || d % 8 || !aligned16(X) || !aligned16(W)) return XFC_ERR_ALIGN;
+  if (ldg < L) return XFC_ERR_SHAPE;
+  if (!ws || ws_bytes < bucket_ws_bytes(L, nnz)) return XFC_ERR_WORKSPACE;
+  BucketWs bk = carve_bucket_ws(ws, L, nnz);
+  const int n_tiles = (int)round_up(ceil_div(L, FwdCore::BN), 8);
+  const bool coo = pos_x != nullptr;
+  hipLaunchKernelGGL(bucket_positives_kernel, dim3(1), dim3(1024), 0, st, coo ? nullptr : rowptr,
+                     coo ? nullptr : colidx, coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L,
+                     FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
+  int rc = check_launch();
+  if (rc) return rc;
+  // label columns L .. min(ldg, round_up(L, 8)) are written as zero so that G can be read in
+  // 16-byte pieces along the label axis by the dX and dW kernels
+  const int64_t n_store = round_up(L, 8) <= ldg ? round_up(L, 8) : L;
+  return launch_fwd(FWD_GRAD, (const half_t*)X, ldx, (const half_t*)W, ldw, (half_t*)G, ldg, (int)B, (int)L, (int)d,
+                    (int)n_store, 1.0f, 0.0f, &bk, st);
+}
+
+int xfc_fwd_grad_csr(const void* X, int64_t ldx, const void* W, int64_t ldw, const int32_t* rowptr,
+                     const int32_t* colidx, void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, int64_t nnz,
+                     void* workspace, size_t workspace_bytes, void* stream) {
+  if (B > 0 && !rowptr) return XFC_ERR_INVALID;
+  return fwd_grad_impl(X, ldx, W, ldw, rowptr, colidx, nullptr, nullptr, nnz, G, ldg, B, L, d, workspace,
+                       workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_fwd_grad_coo(const void* X, int64_t ldx, const void* W, int64_t ldw, const int64_t* pos_x, const int64_t* pos_y,
+                     int64_t nnz, void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  if (nnz > 0 && !(pos_x && pos_y)) return XFC_ERR_INVALID;
+  // an empty list still goes through the bucket pass (it zeroes the bucket table)
+  static const int64_t dummy = 0;
+  return fwd_grad_impl(X, ldx, W, ldw, nullptr, nullptr, pos_x ? pos_x : &dummy, pos_y ? pos_y : &dummy, nnz, G, ldg, B,
+                       L, d, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+size_t xfc_dx_workspace_bytes(int64_t B, int64_t L, int64_t d) { return xfc_gemm_workspace_bytes(B, d, L); }
+
+int xfc_dx(const void* G, int64_t ldg, const void* W, int64_t ldw, float* dX, int64_t lddx, int64_t B, int64_t L,
+           int64_t d, float scale, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
+  if (B == 0 || d == 0) return XFC_OK;
+  if (!G || !W || !dX) return XFC_ERR_INVALID;
+  if (ldg % 8 || ldw % 8 || d % 8 || !aligned16(G) || !aligned16(W)) return XFC_ERR_ALIGN;
+  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
+  return launch_dx((const half_t*)G, ldg, (const half_t*)W, ldw, dX, lddx, (int)B, (int)d, (int)L, scale, 0.0f,
+                   workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_dw_update(const void* G, int64_t ldg, const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int64_t ldm,
+                  int64_t B, int64_t L, int64_t d, float lr, float momentum, float weight_decay, float* dW_out,
+                  int64_t ld_dw, void* stream) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
+  if (L == 0 || d == 0) return XFC_OK;
+  if (!G || !X || !W || !Mo) return XFC_ERR_INVALID;
+  if (ldg % 8 || ldx % 8 || ldw % 8 || ldm % 8 || d % 8 || !aligned16(G) || !aligned16(X) || !aligned16(W) ||
+      !aligned16(Mo))
+    return XFC_ERR_ALIGN;
+  if (dW_out && (ld_dw % 4 || !aligned16(dW_out))) return XFC_ERR_ALIGN;
+  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
+  DwArgs a = {};
+  a.G = (const half_t*)G; a.ldg = ldg; a.X = (const half_t*)X; a.ldx = ldx;
+  a.M = (int)L; a.N = (int)d; a.K = (int)B; a.g_cols = (int)round_up(L, 8);
+  a.Wt = (half_t*)W; a.ldw = ldw; a.Mo = (half_t*)Mo; a.ldm = ldm;
+  a.lr = lr; a.mu = momentum; a.wd = weight_decay; a.dw_dump = dW_out; a.ld_dump = ld_dw;
+  return launch_dw(DW_UPDATE, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_dw(const void* G, int64_t ldg, const void* X, int64_t ldx, float* grad, int64_t ld_grad, int64_t B, int64_t L,
+           int64_t d, float beta, void* stream) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
+  if (L == 0 || d == 0) return XFC_OK;
+  if (!G || !X || !grad) return XFC_ERR_INVALID;
+  if (ldg % 8 || ldx % 8 || d % 8 || ld_grad % 4 || !aligned16(G) || !aligned16(X) || !aligned16(grad))
+    return XFC_ERR_ALIGN;
+  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
+  DwArgs a = {};
+  a.G = (const half_t*)G; a.ldg = ldg; a.X = (const half_t*)X; a.ldx = ldx;
+  a.M = (int)L; a.N = (int)d; a.K = (int)B; a.g_cols = (int)round_up(L, 8);
+  a.out = grad; a.ldo = ld_grad; a.alpha = 1.0f; a.beta = beta;
+  return launch_dw(DW_OUT, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_sgd_momentum(void* W, void* Mo, const float* grad, int64_t count, float lr, float momentum, float weight_decay,
+                     void* stream) {
+  if (count < 0) return XFC_ERR_INVALID;
+  if (count == 0) return XFC_OK;
+  if (!W || !Mo || !grad) return XFC_ERR_INVALID;
+  if (count % 8 || !aligned16(W) || !aligned16(Mo) || !aligned16(grad)) return XFC_ERR_ALIGN;
+  const int64_t n8 = count / 8;
+  hipLaunchKernelGGL(sgd_momentum_kernel, dim3((unsigned)ceil_div(n8, 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), (half_t*)W, (half_t*)Mo, grad, n8, lr, momentum,
+                     weight_decay);
+  return check_launch();
+}
+
+size_t xfc_step_workspace_bytes(int64_t B, int64_t L, int64_t d, int64_t nnz) {
+  return (size_t)round_up(xfc_fwd_grad_workspace_bytes(L, nnz), 256) + xfc_dx_workspace_bytes(B, L, d);
+}
+
+int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int64_t ldm, const int32_t* rowptr,
+                 const int32_t* colidx, int64_t nnz, void* G, int64_t ldg, float* dX, int64_t lddx, int64_t B,
+                 int64_t L, int64_t d, float lr, float momentum, float weight_decay, float scale, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  if (workspace_bytes < xfc_step_workspace_bytes(B, L, d, nnz) || !workspace) return XFC_ERR_WORKSPACE;
+  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
+  const size_t off = (size_t)round_up(xfc_fwd_grad_workspace_bytes(L, nnz), 256);
+  unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
+  int rc = xfc_fwd_grad_csr(X, ldx, W, ldw, rowptr, colidx, G, ldg, B, L, d, nnz, ws, off, stream);
+  if (rc) return rc;
+  rc = xfc_dx(G, ldg, W, ldw, dX, lddx, B, L, d, scale, ws + off, workspace_bytes - off, stream);
+  if (rc) return rc;
+  return xfc_dw_update(G, ldg, X, ldx, W, ldw, Mo, ldm, B, L, d, lr, momentum, weight_decay, nullptr, 0, stream);
+}
+
+}  // extern "C"

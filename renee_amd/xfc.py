@@ -1,0 +1,264 @@
+"""Host side of the XFC layer step: the reference's operator interface for this
+path, driving the HIP kernels through the C ABI (include/xfc_mi355x.h).
+
+  xfc_gemm(...)            the extension function the reference imports as
+                           xfc_gemm_cuda.xfc_gemm (xfc_gemm.cpp:17-40)
+  XFCLayer                 the buffers GenericModel keeps for the classifier
+                           (dl_base.py:175-187) and BCELossMultiNode's
+                           xfc_forward / xfc_backward (dl_base.py:568-642), with
+                           the optimizer step (dl_base.py:343) fused into the dW pass
+
+PyTorch supplies device memory and the current stream; all arithmetic on the
+path is done by the HIP library.
+"""
+from __future__ import annotations
+
+import torch
+
+from ._lib import check, lib
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _round_up(a: int, b: int) -> int:
+    return (a + b - 1) // b * b
+
+
+class _Workspace:
+    """One growable byte buffer per device, handed to calls that need scratch."""
+
+    def __init__(self):
+        self._buf = {}
+
+    def get(self, device: torch.device, nbytes: int) -> torch.Tensor:
+        key = (device.type, device.index)
+        buf = self._buf.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+            self._buf[key] = buf
+        return buf
+
+
+_workspace = _Workspace()
+
+
+def _require(cond: bool, msg: str, exc=RuntimeError):
+    if not cond:
+        raise exc(msg)
+
+
+def xfc_gemm(mat_in1: torch.Tensor, mat_in2: torch.Tensor, mat_out: torch.Tensor,
+             alpha: float, beta: float, apply_sigmoid: bool) -> None:
+    """Drop-in for xfc_gemm_cuda.xfc_gemm (xfc_gemm.cpp:17-23): writes mat_out in
+    place; the GEMM mode follows from the strides of the views passed in
+    (xfc_gemm_kernel.cu:65,113,151).  Unlike the reference, bad arguments raise
+    instead of terminating the process, and dtypes/devices are checked."""
+    for t in (mat_in1, mat_in2, mat_out):
+        _require(t.dim() == 2, "expected 2D tensor")
+        _require(t.is_cuda, "expected a GPU tensor")
+    _require(mat_in1.dtype == torch.float16 and mat_in2.dtype == torch.float16,
+             "mat_in1 and mat_in2 must be float16", TypeError)
+    want = torch.float16 if apply_sigmoid else torch.float32
+    _require(mat_out.dtype == want, f"mat_out must be {want} for apply_sigmoid={bool(apply_sigmoid)}", TypeError)
+    _require(mat_in1.device == mat_in2.device == mat_out.device, "tensors must share a device")
+    M, N = mat_out.shape
+    K = mat_in2.shape[0]
+    L = lib()
+    ws_bytes = L.xfc_gemm_workspace_bytes(M, N, K) if not apply_sigmoid else 0
+    with torch.cuda.device(mat_out.device):
+        ws = _workspace.get(mat_out.device, ws_bytes)
+        rc = L.xfc_gemm(mat_in1.data_ptr(), mat_in1.shape[0], mat_in1.shape[1], mat_in1.stride(0), mat_in1.stride(1),
+                        mat_in2.data_ptr(), mat_in2.shape[0], mat_in2.shape[1], mat_in2.stride(0), mat_in2.stride(1),
+                        mat_out.data_ptr(), M, N, mat_out.stride(0), mat_out.stride(1),
+                        float(alpha), float(beta), int(bool(apply_sigmoid)),
+                        ws.data_ptr(), ws.numel(), _stream(mat_out))
+    check(rc, "xfc_gemm")
+
+
+def coo_to_csr(pos_x: torch.Tensor, pos_y: torch.Tensor, num_rows: int):
+    """Row-sorted COO (dl_base.py:934-936) -> (rowptr int32[B+1], colidx int32[nnz]) on the same device."""
+    counts = torch.bincount(pos_x.long(), minlength=num_rows)
+    rowptr = torch.zeros(num_rows + 1, dtype=torch.int32, device=pos_x.device)
+    rowptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    return rowptr, pos_y.to(torch.int32).contiguous()
+
+
+class XFCLayer:
+    """Label matrix, momentum and scratch buffers of the classifier on one GPU,
+    with the reference's xfc_forward / xfc_backward operators.
+
+    numy is padded as main.py:76-89 does only if the caller asks (pad_to);
+    any label count is accepted.  W and the momentum are fp16 and stay
+    resident; G (`outsoft`, dl_base.py:176) is preallocated for max_batch rows
+    with its rows padded to a multiple of 8 labels.
+    """
+
+    def __init__(self, numy: int, dims: int, max_batch: int, device="cuda:0", lr: float = 0.05,
+                 momentum: float = 0.9, weight_decay: float = 0.0, weight: torch.Tensor | None = None,
+                 seed: int = 0):
+        self.device = torch.device(device)
+        _require(self.device.type == "cuda", "XFCLayer needs a GPU device")
+        _require(dims % 8 == 0, "dims must be a multiple of 8")
+        self.numy, self.dims, self.max_batch = int(numy), int(dims), int(max_batch)
+        self.lr, self.momentum, self.weight_decay = float(lr), float(momentum), float(weight_decay)
+        self.ldg = _round_up(self.numy, 8)
+        if weight is None:
+            g = torch.Generator(device=self.device)
+            g.manual_seed(seed)
+            weight = torch.empty(self.numy, self.dims, device=self.device, dtype=torch.float16)
+            step = 1 << 20
+            for r0 in range(0, self.numy, step):  # N(0, 0.02): dl_base.py:187
+                r1 = min(self.numy, r0 + step)
+                weight[r0:r1] = (torch.randn(r1 - r0, self.dims, generator=g, device=self.device) * 0.02).half()
+        else:
+            _require(tuple(weight.shape) == (self.numy, self.dims), "weight shape")
+            weight = weight.to(device=self.device, dtype=torch.float16).contiguous()
+        self.xfc_weight = weight
+        self.momentum_buffer = torch.zeros_like(self.xfc_weight)
+        self.outsoft = torch.empty(self.max_batch, self.ldg, device=self.device, dtype=torch.float16)
+        self.grad_input = torch.empty(self.max_batch, self.dims, device=self.device, dtype=torch.float32)
+        self.xfc_weight_grad = None  # fp32 accumulator, only under split accumulation
+
+    # -- helpers ---------------------------------------------------------------------------
+    def _x16(self, embed: torch.Tensor) -> torch.Tensor:
+        _require(embed.dim() == 2 and embed.shape[1] == self.dims, "embed must be (batch, dims)")
+        x = embed.to(device=self.device, dtype=torch.float16)  # dl_base.py:561
+        return x if x.stride(1) == 1 and x.stride(0) % 8 == 0 else x.contiguous()
+
+    def _g_view(self, bsz: int) -> torch.Tensor:
+        _require(bsz <= self.max_batch, "batch larger than max_batch")
+        return self.outsoft[0:bsz]
+
+    # -- reference operators ---------------------------------------------------------------
+    def xfc_forward(self, embed: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """Logits out = embed . W^T (dl_base.py:568-573)."""
+        x = self._x16(embed)
+        bsz = x.shape[0]
+        if out is None:
+            out = self._g_view(bsz)[:, : self.numy]
+        _require(out.dtype == torch.float16 and out.stride(1) == 1 and tuple(out.shape) == (bsz, self.numy),
+                 "out must be float16 (batch, numy) with unit column stride")
+        with torch.cuda.device(self.device):
+            rc = lib().xfc_logits(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
+                                  out.data_ptr(), out.stride(0), bsz, self.numy, self.dims, _stream(x))
+        check(rc, "xfc_logits")
+        return out
+
+    def fwd_grad(self, embed, pos_x=None, pos_y=None, rowptr=None, colidx=None) -> torch.Tensor:
+        """G = sigmoid(embed . W^T) - Y into outsoft (dl_base.py:591-594); returns the (batch, numy) view."""
+        x = self._x16(embed)
+        bsz = x.shape[0]
+        G = self._g_view(bsz)
+        L = lib()
+        csr = rowptr is not None
+        nnz = int(colidx.numel() if csr else (0 if pos_x is None else pos_x.numel()))
+        with torch.cuda.device(self.device):
+            ws = _workspace.get(self.device, L.xfc_fwd_grad_workspace_bytes(self.numy, nnz))
+            if csr:
+                _require(rowptr.dtype == torch.int32 and colidx.dtype == torch.int32, "CSR must be int32", TypeError)
+                _require(rowptr.numel() == bsz + 1, "rowptr must have batch+1 entries")
+                rc = L.xfc_fwd_grad_csr(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
+                                        rowptr.data_ptr(), colidx.data_ptr(), G.data_ptr(), self.ldg,
+                                        bsz, self.numy, self.dims, nnz, ws.data_ptr(), ws.numel(), _stream(x))
+            else:
+                if nnz:
+                    _require(pos_x.dtype == torch.int64 and pos_y.dtype == torch.int64, "COO must be int64", TypeError)
+                    _require(pos_x.numel() == pos_y.numel(), "pos_x / pos_y length")
+                    pos_x, pos_y = pos_x.contiguous(), pos_y.contiguous()
+                rc = L.xfc_fwd_grad_coo(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
+                                        pos_x.data_ptr() if nnz else None, pos_y.data_ptr() if nnz else None, nnz,
+                                        G.data_ptr(), self.ldg, bsz, self.numy, self.dims,
+                                        ws.data_ptr(), ws.numel(), _stream(x))
+        check(rc, "xfc_fwd_grad")
+        return G[:, : self.numy]
+
+    def dx(self, bsz: int, grad_input: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+        """grad_input = scale * G . W with W before the update (dl_base.py:602-608)."""
+        if grad_input is None:
+            grad_input = self.grad_input[0:bsz]
+        _require(grad_input.dtype == torch.float32 and grad_input.stride(1) == 1 and
+                 tuple(grad_input.shape) == (bsz, self.dims), "grad_input must be float32 (batch, dims)")
+        L = lib()
+        G = self._g_view(bsz)
+        with torch.cuda.device(self.device):
+            ws = _workspace.get(self.device, L.xfc_dx_workspace_bytes(bsz, self.numy, self.dims))
+            rc = L.xfc_dx(G.data_ptr(), self.ldg, self.xfc_weight.data_ptr(), self.dims, grad_input.data_ptr(),
+                          grad_input.stride(0), bsz, self.numy, self.dims, float(scale),
+                          ws.data_ptr(), ws.numel(), _stream(G))
+        check(rc, "xfc_dx")
+        return grad_input
+
+    def dw_update(self, embed, dW_out: torch.Tensor | None = None, lr: float | None = None) -> None:
+        """dW = G^T . embed fused with M = mu*M + dW + wd*W ; W -= lr*M (dl_base.py:620-634 + :343)."""
+        x = self._x16(embed)
+        bsz = x.shape[0]
+        G = self._g_view(bsz)
+        if dW_out is not None:
+            _require(dW_out.dtype == torch.float32 and dW_out.is_contiguous() and
+                     tuple(dW_out.shape) == (self.numy, self.dims), "dW_out must be contiguous float32 (numy, dims)")
+        with torch.cuda.device(self.device):
+            rc = lib().xfc_dw_update(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0),
+                                     self.xfc_weight.data_ptr(), self.dims, self.momentum_buffer.data_ptr(), self.dims,
+                                     bsz, self.numy, self.dims, self.lr if lr is None else float(lr), self.momentum,
+                                     self.weight_decay, None if dW_out is None else dW_out.data_ptr(), self.dims,
+                                     _stream(x))
+        check(rc, "xfc_dw_update")
+
+    def dw_accumulate(self, embed) -> None:
+        """xfc_weight.grad (+)= G^T . embed for one micro-batch (dl_base.py:620-633)."""
+        x = self._x16(embed)
+        bsz = x.shape[0]
+        G = self._g_view(bsz)
+        first = self.xfc_weight_grad is None
+        if first:
+            self.xfc_weight_grad = torch.empty(self.numy, self.dims, device=self.device, dtype=torch.float32)
+        with torch.cuda.device(self.device):
+            rc = lib().xfc_dw(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0), self.xfc_weight_grad.data_ptr(),
+                              self.dims, bsz, self.numy, self.dims, 0.0 if first else 1.0, _stream(x))
+        check(rc, "xfc_dw")
+
+    def optimizer_step(self, lr: float | None = None) -> None:
+        """SGD-momentum on the accumulated fp32 grad, then drop it (dl_base.py:343-344)."""
+        _require(self.xfc_weight_grad is not None, "no accumulated gradient")
+        with torch.cuda.device(self.device):
+            rc = lib().xfc_sgd_momentum(self.xfc_weight.data_ptr(), self.momentum_buffer.data_ptr(),
+                                        self.xfc_weight_grad.data_ptr(), self.numy * self.dims,
+                                        self.lr if lr is None else float(lr), self.momentum, self.weight_decay,
+                                        _stream(self.xfc_weight))
+        check(rc, "xfc_sgd_momentum")
+        self.xfc_weight_grad = None
+
+    def xfc_backward(self, embed_out, pos_x, pos_y, grad_input=None, scale: float = 1.0,
+                     accumulate: bool = False, lr: float | None = None) -> torch.Tensor:
+        """One batch (or micro-batch) of dl_base.py:576-642 under --noloss: G, then
+        grad_input, then dW.  With accumulate=False the optimizer step is fused
+        into the dW pass; with accumulate=True dW is added to the fp32 grad and
+        optimizer_step() finishes the step."""
+        bsz = embed_out.shape[0]
+        self.fwd_grad(embed_out, pos_x, pos_y)
+        gi = self.dx(bsz, grad_input, scale)
+        if accumulate:
+            self.dw_accumulate(embed_out)
+        else:
+            self.dw_update(embed_out, lr=lr)
+        return gi
+
+    def step_csr(self, embed, rowptr, colidx, scale: float = 1.0, lr: float | None = None) -> torch.Tensor:
+        """The whole step through the single C entry point xfc_step_csr."""
+        x = self._x16(embed)
+        bsz = x.shape[0]
+        G = self._g_view(bsz)
+        gi = self.grad_input[0:bsz]
+        L = lib()
+        nnz = int(colidx.numel())
+        with torch.cuda.device(self.device):
+            ws = _workspace.get(self.device, L.xfc_step_workspace_bytes(bsz, self.numy, self.dims, nnz))
+            rc = L.xfc_step_csr(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
+                                self.momentum_buffer.data_ptr(), self.dims, rowptr.data_ptr(), colidx.data_ptr(), nnz,
+                                G.data_ptr(), self.ldg, gi.data_ptr(), self.dims, bsz, self.numy, self.dims,
+                                self.lr if lr is None else float(lr), self.momentum, self.weight_decay, float(scale),
+                                ws.data_ptr(), ws.numel(), _stream(x))
+        check(rc, "xfc_step_csr")
+        return gi
