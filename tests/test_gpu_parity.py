@@ -1,0 +1,261 @@
+"""Parity of the HIP path (called through the C ABI) with the CPU oracle on the
+same seeded inputs.  The oracle receives the fp16-rounded X and W upcast to
+fp32, so input quantisation is not charged to the kernels.
+
+Tolerance (stated by the task): relative Frobenius error <= 1e-3 on G, dW and
+dX; the same bound is used for W and M after the update (one fp16 rounding of
+each per step)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import xfc_oracle as O
+from renee_amd import XFCLayer, coo_to_csr, synth, xfc_gemm
+from renee_amd._lib import XfcError
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def rel(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float((a - b).norm() / b.norm())
+
+
+def _problem(B, L, d, kmax=8, kmean=2.3, zipf=1.1, seed=0):
+    X = synth.make_X(B, d, seed).half()
+    W = synth.make_W(L, d, seed).half()
+    P = synth.make_positives(B, L, kmax, kmean, zipf, seed)
+    return X, W, P
+
+
+def _check_step(dev, X, W, px, py, lr=0.05, mu=0.9, wd=0.0, scale=1.0, steps=1, csr=None):
+    B, d = X.shape
+    L = W.shape[0]
+    lay = XFCLayer(L, d, B, dev, lr=lr, momentum=mu, weight_decay=wd, weight=W)
+    Xd = X.to(dev)
+    Wo, Mo = W.float(), torch.zeros(L, d)
+    for s in range(steps):
+        print(f"step {s}: B={B} L={L} d={d} nnz={len(px)}", flush=True)
+        ref = O.step(X.float(), Wo, Mo, px, py, lr, mu, wd, scale)
+        if csr is not None:
+            G = lay.fwd_grad(Xd, rowptr=csr[0].to(dev), colidx=csr[1].to(dev))
+        else:
+            G = lay.fwd_grad(Xd, px.to(dev), py.to(dev))
+        assert rel(G, ref["G"]) <= TOL
+        if lay.ldg > L:  # pad columns are written as zero
+            assert float(lay.outsoft[:B, L:].abs().max()) == 0.0
+        # every positive is negative in G, everything else is in (0, 1)
+        Gc = G.float().cpu()
+        mask = torch.zeros(B, L, dtype=torch.bool)
+        if len(px):
+            ok = (px >= 0) & (px < B) & (py >= 0) & (py < L)
+            mask[px[ok], py[ok]] = True
+        assert (Gc[mask] <= 0).all() and (Gc[~mask] >= 0).all()
+        dX = lay.dx(B, scale=scale)
+        assert rel(dX, ref["dX"]) <= TOL
+        dW = torch.empty(L, d, device=dev, dtype=torch.float32)
+        lay.dw_update(Xd, dW_out=dW)
+        assert rel(dW, ref["dW"]) <= TOL
+        # update parity is judged from the same starting point: the oracle is advanced from the
+        # device's fp16 state so that per-step rounding does not compound in the comparison
+        assert rel(lay.xfc_weight, ref["W"]) <= TOL
+        assert rel(lay.momentum_buffer, ref["M"]) <= TOL
+        Wo, Mo = lay.xfc_weight.float().cpu(), lay.momentum_buffer.float().cpu()
+    return lay
+
+
+def test_cfg0_shape(dev):
+    c = synth.CONFIGS[0]
+    X, W, P = _problem(c["B"], c["L"], 768, c["kmax"], c["kmean"], c["zipf"])
+    px, py = P.coo()
+    _check_step(dev, X, W, px, py, steps=2)
+
+
+def test_cfg1_shape_csr(dev):
+    c = synth.CONFIGS[1]
+    X, W, P = _problem(c["B"], c["L"], 768, c["kmax"], c["kmean"], c["zipf"], seed=1)
+    px, py = P.coo()
+    _check_step(dev, X, W, px, py, csr=(torch.from_numpy(P.rowptr), torch.from_numpy(P.colidx)), scale=4096.0)
+
+
+@pytest.mark.parametrize("B,L,d", [(1, 9, 8), (7, 1000, 64), (100, 4097, 128), (264, 12345, 384), (513, 2049, 1024),
+                                   (512, 8313, 768)])
+def test_ragged_shapes(dev, B, L, d):
+    X, W, P = _problem(B, L, d, seed=B)
+    px, py = P.coo()
+    _check_step(dev, X, W, px, py, wd=1e-3, scale=3.0)
+
+
+def test_adversarial_label_sets(dev):
+    B, L, d = 300, 1000 + 121, 64
+    X, W, _ = _problem(B, L, d, seed=9)
+    rows, cols = [], []
+    rows += [5, 5, 5]; cols += [17, 17, 17]                  # duplicated pair counts once
+    rows += list(range(B)); cols += [0] * B                   # a head label positive for every row
+    rows += [0, 299, 256, 255]; cols += [L - 1, L - 1, L - 1, 1024]  # last ragged label tile, tile edges
+    rows += [10, 11]; cols += [127, 128]
+    perm = np.random.default_rng(0).permutation(len(rows))    # unsorted COO
+    px = torch.tensor(rows)[perm]
+    py = torch.tensor(cols)[perm]
+    _check_step(dev, X, W, px, py)
+    # out-of-range pairs are ignored
+    px2 = torch.cat([px, torch.tensor([B, -1, 3])])
+    py2 = torch.cat([py, torch.tensor([0, 0, L])])
+    lay = XFCLayer(L, d, B, dev, weight=W)
+    G2 = lay.fwd_grad(X.to(dev), px2.to(dev), py2.to(dev)).clone()
+    G1 = lay.fwd_grad(X.to(dev), px.to(dev), py.to(dev))
+    assert torch.equal(G1, G2)
+    # no positives at all: G = sigmoid(Z)
+    G0 = lay.fwd_grad(X.to(dev))
+    assert rel(G0, torch.sigmoid(O.logits(X.float(), W.float()))) <= TOL
+
+
+def test_golden_vectors(dev):
+    z = np.load(os.path.join(GOLD, "xfc_step_small.npz"))
+    lr, mu, wd, scale = [float(v) for v in z["hyper"]]
+    X, W = torch.from_numpy(z["X"]).half(), torch.from_numpy(z["W0"]).half()
+    px, py = torch.from_numpy(z["pos_x"]), torch.from_numpy(z["pos_y"])
+    B, d = X.shape
+    L = W.shape[0]
+    lay = XFCLayer(L, d, B, dev, lr=lr, momentum=mu, weight_decay=wd, weight=W)
+    G = lay.fwd_grad(X.to(dev), px.to(dev), py.to(dev))
+    assert rel(G, torch.from_numpy(z["G1"])) <= TOL
+    assert rel(lay.dx(B, scale=scale), torch.from_numpy(z["dX1"])) <= TOL
+    dW = torch.empty(L, d, device=dev)
+    lay.dw_update(X.to(dev), dW_out=dW)
+    assert rel(dW, torch.from_numpy(z["dW1"])) <= TOL
+    assert rel(lay.xfc_weight, torch.from_numpy(z["W1"])) <= TOL
+    assert rel(lay.momentum_buffer, torch.from_numpy(z["M1"])) <= TOL
+    # second step: compounding of two fp16-stored updates stays inside the same bound here
+    lay.xfc_backward(X.to(dev), px.to(dev), py.to(dev), scale=scale)
+    assert rel(lay.xfc_weight, torch.from_numpy(z["W2"])) <= 2 * TOL
+    assert rel(lay.momentum_buffer, torch.from_numpy(z["M2"])) <= 2 * TOL
+
+
+def test_real_label_distribution(dev):
+    """First 256 rows of the reference's LF-AmazonTitles-131K test label matrix
+    (L = 131,073, not a multiple of 8)."""
+    lines = open(os.path.join(GOLD, "lf_amazontitles_131k_tst_first256.txt")).read().splitlines()
+    B, L = [int(v) for v in lines[0].split()]
+    rows, cols = [], []
+    for b, line in enumerate(lines[1:]):
+        for tok in line.split():
+            rows.append(b)
+            cols.append(int(tok.split(":")[0]))
+    px, py = torch.tensor(rows), torch.tensor(cols)
+    assert B == 256 and L == 131073 and len(px) > 256
+    X, W = synth.make_X(B, 768, 5).half(), synth.make_W(L, 768, 5).half()
+    rp, ci = coo_to_csr(px, py, B)
+    _check_step(dev, X, W, px, py, csr=(rp, ci))
+
+
+def test_step_entry_point_and_linearity(dev):
+    B, L, d = 128, 5000, 256
+    X, W, P = _problem(B, L, d, seed=4)
+    rp, ci = torch.from_numpy(P.rowptr).to(dev), torch.from_numpy(P.colidx).to(dev)
+    a = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=1e-4, weight=W)
+    b = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=1e-4, weight=W)
+    px, py = P.coo()
+    for _ in range(3):
+        ga = a.step_csr(X.to(dev), rp, ci, scale=2.0).clone()
+        gb = b.xfc_backward(X.to(dev), px.to(dev), py.to(dev), scale=1.0)
+        assert torch.equal(a.xfc_weight, b.xfc_weight) and torch.equal(a.momentum_buffer, b.momentum_buffer)
+        assert torch.allclose(ga, 2.0 * gb, rtol=1e-6, atol=0)  # dX is linear in the loss scale
+
+
+def test_split_accumulation(dev):
+    """--accum: micro-batches of rows, dW accumulated in fp32, one optimizer step (dl_base.py:318-344)."""
+    B, L, d, xfcz = 200, 3000, 128, 64
+    X, W, P = _problem(B, L, d, seed=6)
+    px, py = P.coo()
+    lay = XFCLayer(L, d, xfcz, dev, lr=0.05, momentum=0.9, weight_decay=1e-3, weight=W)
+    # the collator's layout: pos_x local to each micro-batch, `index` the nnz offsets
+    index, px_local = [0], px.clone()
+    for s in range(0, B, xfcz):
+        e = min(B, s + xfcz)
+        index.append(int(P.rowptr[e]))
+        px_local[index[-2]:index[-1]] -= s
+    gi = torch.empty(B, d, device=dev)
+    for i, s in enumerate(range(0, B, xfcz)):
+        e = min(B, s + xfcz)
+        sl = slice(index[i], index[i + 1])
+        lay.xfc_backward(X[s:e].to(dev), px_local[sl].to(dev), py[sl].to(dev), grad_input=gi[s:e], scale=2.0,
+                         accumulate=True)
+    grad = lay.xfc_weight_grad.clone()
+    lay.optimizer_step()
+    ref = O.step_accum(X.float(), W.float(), torch.zeros(L, d), px_local, py, torch.tensor(index), xfcz,
+                       0.05, 0.9, 1e-3, 2.0)
+    assert rel(gi, ref["dX"]) <= TOL and rel(grad, ref["dW"]) <= TOL
+    assert rel(lay.xfc_weight, ref["W"]) <= TOL and rel(lay.momentum_buffer, ref["M"]) <= TOL
+    assert lay.xfc_weight_grad is None
+
+
+def test_lr_zero_still_updates_momentum(dev):
+    B, L, d = 64, 512, 64
+    X, W, P = _problem(B, L, d, seed=2)
+    px, py = P.coo()
+    lay = XFCLayer(L, d, B, dev, lr=0.0, momentum=0.9, weight=W)
+    lay.xfc_backward(X.to(dev), px.to(dev), py.to(dev))
+    assert torch.equal(lay.xfc_weight.cpu(), W)
+    assert float(lay.momentum_buffer.abs().sum()) > 0
+
+
+def test_xfc_gemm_three_modes(dev):
+    """The reference's call sites: dl_base.py:591, :623, :629 and the dead :604."""
+    B, L, d = 256, 4096, 768
+    X, W, _ = _problem(B, L, d, seed=3)
+    Xd, Wd = X.to(dev), W.to(dev)
+    out = torch.full((B, L), float("nan"), device=dev, dtype=torch.float16)  # beta = 0 must not read it
+    xfc_gemm(Xd, Wd.t(), out, 1.0, 0.0, True)
+    ref = X.float().clone(), W.float().clone()
+    want = torch.sigmoid(O.logits(*ref))
+    assert rel(out, want) <= TOL
+    G = out
+    grad = torch.full((L, d), float("nan"), device=dev)
+    xfc_gemm(G.t(), Xd, grad, 1.0, 0.0, False)
+    want_dw = O.dw(G.float().cpu(), X.float())
+    assert rel(grad, want_dw) <= TOL
+    xfc_gemm(G.t(), Xd, grad, 1.0, 1.0, False)
+    assert rel(grad, 2 * want_dw) <= TOL
+    gi = torch.full((B, d), float("nan"), device=dev)
+    xfc_gemm(G, Wd, gi, 4096.0, 0.0, False)
+    assert rel(gi, O.dx(G.float().cpu(), W.float(), 4096.0)) <= TOL
+    # alpha / beta on the sigmoid mode
+    prev = (torch.randn(B, L) * 0.5).half()
+    out2 = prev.to(dev)
+    xfc_gemm(Xd, Wd.t(), out2, 2.0, 0.5, True)
+    assert rel(out2, torch.sigmoid(2.0 * O.logits(*ref) + 0.5 * prev.float())) <= TOL
+
+
+def test_xfc_gemm_any_stride_fallback_and_errors(dev):
+    B, L, d = 9, 37, 20  # nothing is a multiple of 8
+    g = torch.Generator().manual_seed(0)
+    X, W = torch.randn(B, d, generator=g).half(), (torch.randn(L, d, generator=g) * 0.2).half()
+    Xd, Wd = X.to(dev), W.to(dev)
+    out = torch.empty(B, L, device=dev, dtype=torch.float16)
+    xfc_gemm(Xd, Wd.t(), out, 1.0, 0.0, True)
+    assert rel(out, torch.sigmoid(O.logits(X.float(), W.float()))) <= TOL
+    grad = torch.empty(L, d, device=dev)
+    xfc_gemm(out.t(), Xd, grad, 1.0, 0.0, False)
+    assert rel(grad, O.dw(out.float().cpu(), X.float())) <= TOL
+    gi = torch.empty(B, d, device=dev)
+    xfc_gemm(out, Wd, gi, 2.0, 0.0, False)
+    assert rel(gi, O.dx(out.float().cpu(), W.float(), 2.0)) <= TOL
+    with pytest.raises(XfcError):  # row x row with apply_sigmoid: the reference exits the process here
+        xfc_gemm(Xd, Wd.t().contiguous(), out, 1.0, 0.0, True)
+    with pytest.raises(XfcError):  # inner dimensions disagree
+        xfc_gemm(Xd[:, :8], Wd.t(), out, 1.0, 0.0, True)
+    with pytest.raises(TypeError):
+        xfc_gemm(Xd.float(), Wd.t(), out, 1.0, 0.0, True)
+
+
+def test_logits(dev):
+    B, L, d = 130, 3001, 768
+    X, W, _ = _problem(B, L, d, seed=8)
+    lay = XFCLayer(L, d, B, dev, weight=W)
+    Z = lay.xfc_forward(X.to(dev))
+    assert rel(Z, O.logits(X.float(), W.float())) <= TOL
