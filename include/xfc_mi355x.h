@@ -66,6 +66,7 @@ int xfc_gemm(const void* in1, int64_t in1_rows, int64_t in1_cols, int64_t in1_s0
 /*
  * Logits only: out[B x L] (fp16) = X[B x d] . W[L x d]^T.
  * Replaces BCELossMultiNode.xfc_forward, dl_base.py:568-573 (torch.matmul(out=)).
+ * ldx, ldw, ldo and d must be multiples of 8 and the pointers 16-byte aligned.
  */
 int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out, int64_t ldo,
                int64_t B, int64_t L, int64_t d, void* stream);
@@ -79,7 +80,7 @@ int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out
  * are ignored.  Positives come either as CSR (rowptr int32[B+1], colidx
  * int32[nnz]) or as the reference's COO pair (pos_x, pos_y int64[nnz],
  * dl_base.py:934-936), in any order.
- * G has leading dimension ldg >= L; when ldg >= round_up(L, 8) the columns
+ * G has leading dimension ldg >= L, a multiple of 8; the columns
  * L .. round_up(L,8)-1 are written as zero (xfc_dx / xfc_dw_update rely on it).
  * Workspace: xfc_fwd_grad_workspace_bytes(L, nnz) bytes.
  */

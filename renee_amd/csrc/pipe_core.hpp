@@ -1,0 +1,394 @@
+// Multi-stage fp16 MFMA main loop for gfx950 (CDNA4) with direct global->LDS loads.
+//
+// One workgroup of WM x WN wavefronts owns a BM x BN accumulator tile and walks the
+// contraction index in steps of BK.  Operand tiles travel HBM/L2 -> LDS without passing
+// through registers (global_load_lds_dwordx4: every lane fetches 16 bytes from its own
+// address and the wave's 64 pieces land in 1 KB of consecutive LDS).  STAGES tile pairs
+// are resident; STAGES-1 are in flight ahead of the one being multiplied, and the ring keeps
+// turning across the tiles a workgroup processes, so a tile's epilogue runs with the next
+// tile's operands already on their way.
+//
+// Operand storage in global memory:
+//   KC ("K-contiguous"):  elem(r, k) at P[r*ld + k]     LDS: [r][BK], 16-byte chunks XOR-swizzled by row
+//   MC ("M/N-contiguous"): elem(r, k) at P[k*ld + r]    LDS: [k][R],  16-byte chunks XOR-swizzled by k
+// KC fragments are read with ds_read_b128, MC fragments with ds_read_b64_tr_b16.
+// Pieces outside the operand (row, column or k past its limit) are fetched from a 16-byte
+// block of zeros instead, so every LDS slot is always written.
+//
+// MFMA 32x32x16 register layout (checked on hardware):
+//   A: lane l holds A[i = l%32][k = 8*(l/32) .. +7]
+//   B: lane l holds B[k = 8*(l/32) .. +7][j = l%32]
+//   C: lane l, register r holds C[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32]
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xfc {
+
+typedef _Float16 half_t;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+#define XFC_LDS __attribute__((address_space(3)))
+#define XFC_GLB __attribute__((address_space(1)))
+
+__device__ __attribute__((aligned(16))) const uint32_t g_zero16[4] = {0u, 0u, 0u, 0u};
+
+// Row of C held by accumulator register r of a 32x32 block, for this lane.
+__device__ __forceinline__ int c_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// Waits until at most N of this wave's vector-memory operations are outstanding, then joins the
+// workgroup barrier.  Written as one asm block: a plain __syncthreads() carries a fence that makes
+// the compiler drain every outstanding global->LDS fetch first, which would serialise the ring.
+// The "memory" clobber keeps the compiler from moving LDS or global accesses across it.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_lds_vmcnt_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// 16 bytes per lane from `g` to LDS at lds_base + lane*16 (lds_base wave-uniform).
+__device__ __forceinline__ void load16_to_lds(const void* g, void* lds_base) {
+  __builtin_amdgcn_global_load_lds((XFC_GLB const void*)g, (XFC_LDS void*)lds_base, 16, 0, 0);
+}
+
+template <int BK>
+__device__ __forceinline__ int kc_swz(int row) {
+  // ds_read_b128 is served 16 lanes at a time over 64 banks: the 16 rows one group reads must spread
+  // over all 256 bytes.  Measured: 212 B/clk/CU (BK 64) and 220 (BK 32), against 63-122 for other choices.
+  if constexpr (BK == 64) return (row >> 1) & 7;
+  else return (row >> 2) & 3;
+}
+// MC tiles: chunk index within a k-row is XORed with 4*(k%4): the four k-rows one
+// transposing read touches then sit in four different 64-byte bank groups.
+__device__ __forceinline__ int mc_swz(int k) { return (k & 3) << 2; }
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_, int PF_ = 3>
+struct PipeCore {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
+  static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
+  static constexpr int NW = WM * WN, NT = 64 * NW;
+  static constexpr int TM = BM / WM, TN = BN / WN;
+  static constexpr int FM = TM / 32, FN = TN / 32;
+  static constexpr int CPR = BK / 8;
+  static constexpr int A_HALVES = BM * BK, B_HALVES = BN * BK;
+  static constexpr int STAGE_HALVES = A_HALVES + B_HALVES;
+  static constexpr int RING_BYTES = STAGES * STAGE_HALVES * 2;
+  static constexpr int LDS_BYTES = RING_BYTES + (PF_ > 0 ? WM * WN * 256 : 0);
+  static constexpr int A_CH = BM * BK / 8 / NT, B_CH = BN * BK / 8 / NT;
+  static constexpr int PF = PF_;  // the L2 is warmed this many stages ahead of the LDS fill (0: off)
+  static constexpr int LOADS_PER_STAGE = A_CH + B_CH + (PF > 0 ? 1 : 0);
+  static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile must be 32-multiples");
+  static_assert((BM * BK / 8) % NT == 0 && (BN * BK / 8) % NT == 0, "chunk split");
+  static_assert(BK == 32 || BK == 64, "BK");
+  static_assert(A_KC || BM >= 128, "MC swizzle needs 16 chunks per k-row");
+  static_assert(B_KC || BN >= 128, "MC swizzle needs 16 chunks per k-row");
+  static_assert(STAGES >= 2 && (STAGES - 1) * LOADS_PER_STAGE < 64, "stages");
+
+  struct Operand {
+    const half_t* p;
+    int64_t ld;
+    int r0, rmax, kmax;  // first row (or column) of the tile, its limit, limit of the k index
+  };
+
+  // Per-thread addresses of the CH 16-byte pieces it fetches for one operand each stage.
+  template <bool KC, int R, int CH>
+  struct Loader {
+    const half_t* ptr[CH];
+    int koff[CH];
+    uint32_t ok;
+    int kmax;
+    int64_t kstride;
+    __device__ __forceinline__ void init(const Operand& o, int k_begin, int wave, int lane) {
+      ok = 0u;
+      kmax = o.kmax;
+      kstride = KC ? (int64_t)BK : (int64_t)BK * o.ld;
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        const int q = (i * NW + wave) * 64 + lane;
+        int r, k;
+        if constexpr (KC) {
+          const int row = q / CPR, pc = q % CPR;
+          r = row;
+          k = (pc ^ kc_swz<BK>(row)) * 8;
+        } else {
+          const int krow = q / (R / 8), pc = q % (R / 8);
+          k = krow;
+          r = (pc ^ mc_swz(krow)) * 8;
+        }
+        const int gr = o.r0 + r;
+        if (gr < o.rmax) ok |= 1u << i;
+        koff[i] = k;
+        const int gk = k_begin + k;
+        ptr[i] = KC ? o.p + (int64_t)gr * o.ld + gk : o.p + (int64_t)gk * o.ld + gr;
+      }
+    }
+    // k0: absolute k of the stage being fetched
+    __device__ __forceinline__ void issue(half_t* region, int k0, int wave) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        const bool valid = ((ok >> i) & 1u) && (k0 + koff[i] < kmax);
+        const void* src = valid ? (const void*)ptr[i] : (const void*)g_zero16;
+        load16_to_lds(src, region + (i * NW + wave) * 512);
+        ptr[i] += kstride;
+      }
+    }
+  };
+  using LoaderA = Loader<A_KC, BM, A_CH>;
+  using LoaderB = Loader<B_KC, BN, B_CH>;
+
+  // L2 warm-up: HBM latency (microseconds under load) is longer than the ring can cover, so every
+  // thread touches one 128-byte line of a stage PF stages before that stage's LDS fill is issued
+  // (4 bytes per lane into a scratch corner of LDS).  The first half of the workgroup's threads
+  // walks operand A's lines, the second half operand B's; the fill then finds its data in L2.
+  struct Prefetcher {
+    const half_t* ptr;
+    int koff, kmax;
+    bool ok;
+    int64_t kstride;
+    template <bool KC, int R>
+    __device__ __forceinline__ void init_op(const Operand& o, int k_begin, int u) {
+      kmax = o.kmax;
+      kstride = KC ? (int64_t)BK : (int64_t)BK * o.ld;
+      if constexpr (KC) {
+        const int row = u;  // one line per row when BK == 64 (half a line when 32)
+        ok = u < R && o.r0 + row < o.rmax;
+        koff = 0;
+        ptr = o.p + (int64_t)(o.r0 + row) * o.ld + k_begin;
+      } else {
+        constexpr int LPR = R / 64;  // 128-byte lines per k-row
+        const int krow = u / LPR, seg = u % LPR;
+        ok = u < BK * LPR && o.r0 + seg * 64 < o.rmax;
+        koff = krow;
+        ptr = o.p + (int64_t)(k_begin + krow) * o.ld + o.r0 + seg * 64;
+      }
+    }
+    __device__ __forceinline__ void init(const Operand& oa, const Operand& ob, int k_begin) {
+      const int t = threadIdx.x;
+      if (t < NT / 2) init_op<A_KC, BM>(oa, k_begin, t);
+      else init_op<B_KC, BN>(ob, k_begin, t - NT / 2);
+    }
+    __device__ __forceinline__ void issue(void* lds_scratch, int k0) {
+      const void* src = (ok && k0 + koff < kmax) ? (const void*)ptr : (const void*)g_zero16;
+      __builtin_amdgcn_global_load_lds((XFC_GLB const void*)src, (XFC_LDS void*)lds_scratch, 4, 0, 0);
+      ptr += kstride;
+    }
+  };
+
+  __device__ __forceinline__ static half8 frag_kc(const half_t* lds, int row0, int kk, int lane) {
+    const int r = row0 + (lane & 31);
+    const int c = kk * 2 + (lane >> 5);
+    return *reinterpret_cast<const half8*>(lds + r * BK + ((c ^ kc_swz<BK>(r)) * 8));
+  }
+
+  // 32 columns starting at col0 of an MC tile [k][R]: within each 16-lane group, lane t
+  // supplies the address of row k + t/4, columns c0 + 4*(t%4)..+3 and receives column
+  // c0 + t for four consecutive k.
+  template <int R>
+  __device__ __forceinline__ static half8 frag_mc(const half_t* lds, int col0, int kk, int lane) {
+    const int g = lane >> 4, t = lane & 15;
+    const int k = kk * 16 + 8 * (g >> 1) + (t >> 2);
+    const int c = col0 + 16 * (g & 1) + 4 * (t & 3);
+    const int off = k * R + ((((c >> 3) ^ mc_swz(k)) << 3) | (c & 7));
+    fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16((XFC_LDS fp16x4_t*)(lds + off));
+    fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16((XFC_LDS fp16x4_t*)(lds + off + 4 * R));
+    half8 out;
+    out[0] = (half_t)lo[0]; out[1] = (half_t)lo[1]; out[2] = (half_t)lo[2]; out[3] = (half_t)lo[3];
+    out[4] = (half_t)hi[0]; out[5] = (half_t)hi[1]; out[6] = (half_t)hi[2]; out[7] = (half_t)hi[3];
+    return out;
+  }
+
+  struct Frags {
+    half8 a[FM], b[FN];
+  };
+  __device__ __forceinline__ static void load_frags(const half_t* st, int kk, int wm, int wn, int lane, Frags& f) {
+    const half_t* sa = st;
+    const half_t* sb = st + A_HALVES;
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+      if constexpr (A_KC) f.a[fm] = frag_kc(sa, wm * TM + fm * 32, kk, lane);
+      else f.a[fm] = frag_mc<BM>(sa, wm * TM + fm * 32, kk, lane);
+    }
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+      if constexpr (B_KC) f.b[fn] = frag_kc(sb, wn * TN + fn * 32, kk, lane);
+      else f.b[fn] = frag_mc<BN>(sb, wn * TN + fn * 32, kk, lane);
+    }
+  }
+  __device__ __forceinline__ static void mfma_all(const Frags& f, float16v (&acc)[FM][FN]) {
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int fn = 0; fn < FN; ++fn)
+        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[fm], f.b[fn], acc[fm][fn], 0, 0, 0);
+  }
+
+  __device__ __forceinline__ static void zero(float16v (&acc)[FM][FN]) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  }
+
+  // Walks the work items [item_begin, item_end) of this workgroup.
+  //   get(item, oa, ob, k_begin, k_end)  fills the operands and the k range of an item (k_end > k_begin,
+  //                                      k_begin a multiple of BK)
+  //   epilogue(item, acc)                consumes the finished accumulators; it may use global memory and LDS
+  //                                      outside the ring's LDS_BYTES
+  // All threads of the workgroup call this together.
+  //
+  // Schedule per stage c (BK/16 sub-steps): the operand fragments of sub-step kk+1 are read from LDS
+  // while the MFMAs of sub-step kk run.  Before the MFMAs of the last sub-step the wave waits for its
+  // part of stage c+1 to have landed and joins the barrier; past it, every wave has finished reading
+  // stage c, so its slot is refilled with stage c+STAGES, and the first fragments of stage c+1 are
+  // read under the last MFMAs of stage c.
+  template <class GetItem, class Epilogue>
+  __device__ __forceinline__ static void run(int item_begin, int item_end, half_t* lds, GetItem get, Epilogue epilogue) {
+    if (item_begin >= item_end) return;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    constexpr int KK = BK / 16;
+    float16v acc[FM][FN];
+    zero(acc);
+
+    // warm-up cursor: PF stages ahead of the fill cursor
+    Prefetcher pf;
+    int p_item = item_begin, p_k = 0, p_kend = 0;
+    bool p_live = PF > 0;
+    void* pf_lds = reinterpret_cast<unsigned char*>(lds) + RING_BYTES + wave * 256;
+    if constexpr (PF > 0) {
+      Operand oa, ob;
+      get(p_item, oa, ob, p_k, p_kend);
+      pf.init(oa, ob, p_k);
+    }
+    auto prefetch_one = [&]() {
+      if constexpr (PF > 0) {
+        if (p_live) {
+          pf.issue(pf_lds, p_k);
+          p_k += BK;
+          if (p_k >= p_kend) {
+            ++p_item;
+            if (p_item < item_end) {
+              Operand oa, ob;
+              get(p_item, oa, ob, p_k, p_kend);
+              pf.init(oa, ob, p_k);
+            } else {
+              p_live = false;
+            }
+          }
+        } else {
+          __builtin_amdgcn_global_load_lds((XFC_GLB const void*)g_zero16, (XFC_LDS void*)pf_lds, 4, 0, 0);
+        }
+      }
+    };
+
+    // fill cursor
+    LoaderA la;
+    LoaderB lb;
+    int i_item = item_begin, i_k = 0, i_kend = 0, i_slot = 0;
+    bool i_live = true;
+    {
+      Operand oa, ob;
+      get(i_item, oa, ob, i_k, i_kend);
+      la.init(oa, i_k, wave, lane);
+      lb.init(ob, i_k, wave, lane);
+    }
+    auto issue_one = [&]() {
+      half_t* st = lds + i_slot * STAGE_HALVES;
+      if (i_live) {
+        la.issue(st, i_k, wave);
+        lb.issue(st + A_HALVES, i_k, wave);
+        i_k += BK;
+        if (i_k >= i_kend) {
+          ++i_item;
+          if (i_item < item_end) {
+            Operand oa, ob;
+            get(i_item, oa, ob, i_k, i_kend);
+            la.init(oa, i_k, wave, lane);
+            lb.init(ob, i_k, wave, lane);
+          } else {
+            i_live = false;
+          }
+        }
+      } else {
+        // past the last stage: keep the count of outstanding fetches per iteration constant
+#pragma unroll
+        for (int i = 0; i < A_CH + B_CH; ++i) load16_to_lds((const void*)g_zero16, st + (i * NW + wave) * 512);
+      }
+      i_slot = i_slot + 1 == STAGES ? 0 : i_slot + 1;
+      prefetch_one();  // issued after the fill, so the fill is never behind a younger, slower request
+    };
+    if constexpr (PF > 0) {
+#pragma unroll
+      for (int s = 0; s < PF; ++s) prefetch_one();
+    }
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue_one();
+    wait_vmcnt_barrier<(STAGES - 2) * LOADS_PER_STAGE>();
+    issue_one();
+
+    Frags cur, nxt;
+    load_frags(lds, 0, wm, wn, lane, cur);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    int c_slot = 0;
+    bool drain_all = false;
+    for (int item = item_begin; item < item_end; ++item) {
+      int kb, ke;
+      {
+        Operand oa, ob;
+        get(item, oa, ob, kb, ke);
+      }
+      const int nk = (ke - kb + BK - 1) / BK;
+      for (int kt = 0; kt < nk; ++kt) {
+        const half_t* st = lds + c_slot * STAGE_HALVES;
+#pragma unroll
+        for (int kk = 0; kk + 1 < KK; ++kk) {
+          load_frags(st, kk + 1, wm, wn, lane, nxt);
+          __builtin_amdgcn_sched_barrier(0);
+          mfma_all(cur, acc);
+          __builtin_amdgcn_sched_barrier(0);
+          cur = nxt;
+        }
+        const int n_slot = c_slot + 1 == STAGES ? 0 : c_slot + 1;
+        // this wave's LDS reads of stage c are complete (lgkmcnt) and its share of stage c+1 has landed.
+        // After an epilogue the wave's stores share the counter with the fetches and may retire out of
+        // order with them, so the first wait after one drains everything.
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0), in a form the compiler's own wait bookkeeping sees
+        if (drain_all) { wait_lds_vmcnt_barrier<0>(); drain_all = false; }
+        else wait_lds_vmcnt_barrier<(STAGES - 2) * LOADS_PER_STAGE>();
+        issue_one();  // stage c + STAGES into the slot of stage c
+        load_frags(lds + n_slot * STAGE_HALVES, 0, wm, wn, lane, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_all(cur, acc);
+        __builtin_amdgcn_sched_barrier(0);
+        // No LDS read stays pending across the loop edge (the reads above finished long before the
+        // MFMAs were all issued): the compiler then knows the next stage's first MFMAs need no wait.
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        cur = nxt;
+        c_slot = n_slot;
+      }
+      epilogue(item, acc);
+      zero(acc);
+      drain_all = true;
+    }
+    wait_vmcnt<0>();
+  }
+};
+
+}  // namespace xfc

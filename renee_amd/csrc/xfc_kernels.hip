@@ -9,7 +9,7 @@
 #include <stdio.h>
 
 #include "../../include/xfc_mi355x.h"
-#include "gemm_core.hpp"
+#include "pipe_core.hpp"
 
 namespace xfc {
 
@@ -105,8 +105,10 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
 // ---------------------------------------------------------------------------------------------
 enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2 };
 
-using FwdCore = GemmCore<256, 128, 64, 2, 2, true, true>;
-constexpr int FWD_LDS_BYTES = FwdCore::STAGE_HALVES * 2;
+using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true, 0>;
+constexpr int FWD_AUX_BYTES = FwdCore::BN * (FwdCore::BM / 32) * 4;  // bitmap, then 8 x 64 halves of staging per wave
+static_assert(FWD_AUX_BYTES >= FwdCore::NW * 512 * 2 && FwdCore::FN == 2, "staging fits the bitmap area");
+constexpr int FWD_LDS_BYTES = FwdCore::LDS_BYTES + FWD_AUX_BYTES;
 
 struct FwdArgs {
   const half_t* X; int64_t ldx;     // M x K, K-contiguous
@@ -115,82 +117,112 @@ struct FwdArgs {
   int M, N, K, n_store;             // columns N <= c < n_store are written as zero
   float alpha, beta;
   const int32_t* bucket_ptr; const int32_t* ent_row; const int32_t* ent_col;
-  int tiles_m, tiles_n;
+  int tiles_m, tiles_n, n_ids;      // n_ids = tiles_m * round_up(tiles_n, 8)
 };
 
-template <int MODE>
-__global__ void __launch_bounds__(256, 2) fwd_kernel(FwdArgs a) {
+// Persistent: workgroup w takes tile ids w, w + gridDim.x, ... (gridDim.x a multiple of 8, so an
+// id keeps its XCD and the row tiles of one label tile run side by side on one L2).
+template <int MODE, bool BETA>
+__global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
   using C = FwdCore;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
-  int mt, nt;
-  xcd_map(blockIdx.x, a.tiles_m, mt, nt);
-  if (nt >= a.tiles_n) return;
-  const int m0 = mt * C::BM, n0 = nt * C::BN;
-  float16v acc[C::FM][C::FN];
-#pragma unroll
-  for (int i = 0; i < C::FM; ++i)
-#pragma unroll
-    for (int j = 0; j < C::FN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  typename C::Operand oa{a.X, a.ldx, m0, a.M, a.K};
-  typename C::Operand ob{a.W, a.ldw, n0, a.N, a.K};
-  C::template run<1>(oa, ob, 0, a.K, lds, acc);
-
+  // 4 KB beside the ring: first the tile's positives bitmap, then per-wave store staging
+  uint32_t* bm = reinterpret_cast<uint32_t*>(smem_raw + C::LDS_BYTES);
+  const int G = gridDim.x, w = blockIdx.x;
+  const int n_items = (a.n_ids - w + G - 1) / G;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
-  // positives of this tile -> bitmap [label][row word]
-  uint32_t* bm = reinterpret_cast<uint32_t*>(smem_raw);
-  bool has = false;
-  if constexpr (MODE == FWD_GRAD) {
-    const int s = a.bucket_ptr[nt], e = a.bucket_ptr[nt + 1];
-    has = e > s;
-    if (has) {
-      for (int i = threadIdx.x; i < C::BN * (C::BM / 32); i += C::NT) bm[i] = 0u;
-      __syncthreads();
-      for (int p = s + threadIdx.x; p < e; p += C::NT) {
-        const int r = a.ent_row[p] - m0, c = a.ent_col[p] - n0;
-        if (r >= 0 && r < C::BM) atomicOr(&bm[c * (C::BM / 32) + (r >> 5)], 1u << (r & 31));
+  half_t* stg = reinterpret_cast<half_t*>(bm) + wave * 512;  // 8 rows x 64 labels
+
+  auto get = [&](int item, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
+    int mt, nt;
+    xcd_map(item * G + w, a.tiles_m, mt, nt);
+    oa = typename C::Operand{a.X, a.ldx, mt * C::BM, a.M, a.K};
+    ob = typename C::Operand{a.W, a.ldw, nt * C::BN, nt < a.tiles_n ? a.N : 0, a.K};
+    kb = 0;
+    ke = a.K;
+  };
+  auto epilogue = [&](int item, float16v (&acc)[C::FM][C::FN]) {
+    int mt, nt;
+    xcd_map(item * G + w, a.tiles_m, mt, nt);
+    if (nt >= a.tiles_n) return;
+    const int m0 = mt * C::BM, n0 = nt * C::BN;
+    // positives of this tile -> bitmap [label][row word] -> one word per 32x32 block and lane
+    uint32_t words[C::FM][C::FN];
+#pragma unroll
+    for (int fm = 0; fm < C::FM; ++fm)
+#pragma unroll
+      for (int fn = 0; fn < C::FN; ++fn) words[fm][fn] = 0u;
+    if constexpr (MODE == FWD_GRAD) {
+      const int s = a.bucket_ptr[nt], e = a.bucket_ptr[nt + 1];
+      if (e > s) {
+        __syncthreads();  // every wave is done staging the previous tile
+        for (int i = threadIdx.x; i < C::BN * (C::BM / 32); i += C::NT) bm[i] = 0u;
+        __syncthreads();
+        for (int p = s + threadIdx.x; p < e; p += C::NT) {
+          const int r = a.ent_row[p] - m0, c = a.ent_col[p] - n0;
+          if (r >= 0 && r < C::BM) atomicOr(&bm[c * (C::BM / 32) + (r >> 5)], 1u << (r & 31));
+        }
+        __syncthreads();
+#pragma unroll
+        for (int fm = 0; fm < C::FM; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < C::FN; ++fn)
+            words[fm][fn] = bm[(wn * C::TN + fn * 32 + (lane & 31)) * (C::BM / 32) + ((wm * C::TM + fm * 32) >> 5)];
+        __syncthreads();  // bitmap consumed: the area is staging again
       }
-      __syncthreads();
     }
-  }
+    const int h = lane >> 5;
+    const int srow = lane >> 3, sch = lane & 7;          // staging read: 8 rows x 8 chunks of 8 labels
+    const int col = n0 + wn * C::TN + sch * 8;
 #pragma unroll
-  for (int fm = 0; fm < C::FM; ++fm) {
+    for (int fm = 0; fm < C::FM; ++fm) {
 #pragma unroll
-    for (int fn = 0; fn < C::FN; ++fn) {
-      const int lcol = wn * C::TN + fn * 32 + (lane & 31);
-      const int col = n0 + lcol;
-      uint32_t word = 0u;
-      if constexpr (MODE == FWD_GRAD) {
-        if (has) word = bm[lcol * (C::BM / 32) + ((wm * C::TM + fm * 32) >> 5)];
-      }
-      if (col < a.n_store) {
+      for (int q = 0; q < 4; ++q) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int lr = c_row(r, lane);
-          const int row = m0 + wm * C::TM + fm * 32 + lr;
-          if (row < a.M) {
-            half_t* dst = a.out + (int64_t)row * a.ldo + col;
+        for (int fn = 0; fn < C::FN; ++fn) {
+          const int ecol = n0 + wn * C::TN + fn * 32 + (lane & 31);
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const int r = 4 * q + rr;
             float v = a.alpha * acc[fm][fn][r];
-            if (a.beta != 0.f) v += a.beta * (float)(*dst);
+            if constexpr (BETA) {
+              const int erow = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
+              if (erow < a.M && ecol < a.N) v += a.beta * (float)a.out[(int64_t)erow * a.ldo + ecol];
+            }
             if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
-            if constexpr (MODE == FWD_GRAD) v -= (float)((word >> lr) & 1u);
-            if (col >= a.N) v = 0.f;
-            *dst = (half_t)v;
+            if constexpr (MODE == FWD_GRAD) v -= (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
+            if (ecol >= a.N) v = 0.f;
+            stg[(4 * h + rr) * 64 + fn * 32 + (lane & 31)] = (half_t)v;
+          }
+        }
+        // the wave's LDS traffic is ordered: its own writes above are visible to the read below
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        const half8 v8 = *reinterpret_cast<const half8*>(stg + srow * 64 + sch * 8);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
+        if (row < a.M) {
+          half_t* dst = a.out + (int64_t)row * a.ldo + col;
+          if (col + 8 <= a.n_store) {
+            *reinterpret_cast<half8*>(dst) = v8;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (col + e < a.n_store) dst[e] = v8[e];
           }
         }
       }
     }
-  }
+  };
+  C::run(0, n_items, lds, get, epilogue);
 }
 
 // ---------------------------------------------------------------------------------------------
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
-using DxCore = GemmCore<256, 128, 64, 2, 2, true, false>;
-constexpr int DX_LDS_BYTES = DxCore::STAGE_HALVES * 2;
+using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, 0>;
+constexpr int DX_LDS_BYTES = DxCore::LDS_BYTES;
 
 struct DxArgs {
   const half_t* G; int64_t ldg;   // M x K, K-contiguous (K = labels)
@@ -200,44 +232,50 @@ struct DxArgs {
   int tiles_m, tiles_n, splits, k_per_split;  // k_per_split is a multiple of BK
 };
 
-__global__ void __launch_bounds__(256, 2) dx_kernel(DxArgs a) {
+// One workgroup per (output tile, slice of the label axis); the tiles of one slice get ids on one XCD.
+__global__ void __launch_bounds__(DxCore::NT) dx_kernel(DxArgs a) {
   using C = DxCore;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
   int tile, split;
   xcd_map(blockIdx.x, a.tiles_m * a.tiles_n, tile, split);
-  if (split >= a.splits) return;
   const int mt = tile % a.tiles_m, nt = tile / a.tiles_m;
   const int m0 = mt * C::BM, n0 = nt * C::BN;
-  float16v acc[C::FM][C::FN];
-#pragma unroll
-  for (int i = 0; i < C::FM; ++i)
-#pragma unroll
-    for (int j = 0; j < C::FN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  const int64_t kb = (int64_t)split * a.k_per_split;
-  const int k_begin = (int)(kb < a.K ? kb : a.K);
-  const int k_end = (int)(kb + a.k_per_split < a.K ? kb + a.k_per_split : a.K);
-  typename C::Operand oa{a.G, a.ldg, m0, a.M, a.K};
-  typename C::Operand ob{a.W, a.ldw, n0, a.N, a.K};
-  C::template run<1>(oa, ob, k_begin, k_end, lds, acc);
+  const int64_t kb64 = (int64_t)split * a.k_per_split;
+  const int k_begin = (int)(kb64 < a.K ? kb64 : a.K);
+  const int k_end = (int)(kb64 + a.k_per_split < a.K ? kb64 + a.k_per_split : a.K);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
   float* part = a.part + (int64_t)split * a.M * a.N;
+  auto store = [&](float16v (&acc)[C::FM][C::FN]) {
 #pragma unroll
-  for (int fm = 0; fm < C::FM; ++fm)
+    for (int fm = 0; fm < C::FM; ++fm)
 #pragma unroll
-    for (int fn = 0; fn < C::FN; ++fn) {
-      const int col = n0 + wn * C::TN + fn * 32 + (lane & 31);
-      if (col < a.N) {
+      for (int fn = 0; fn < C::FN; ++fn) {
+        const int col = n0 + wn * C::TN + fn * 32 + (lane & 31);
+        if (col < a.N) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
-          if (row < a.M) part[(int64_t)row * a.N + col] = acc[fm][fn][r];
+          for (int r = 0; r < 16; ++r) {
+            const int row = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
+            if (row < a.M) part[(int64_t)row * a.N + col] = acc[fm][fn][r];
+          }
         }
       }
-    }
+  };
+  if (k_end <= k_begin) {  // a slice past the end of the label axis contributes zeros
+    float16v acc[C::FM][C::FN];
+    C::zero(acc);
+    store(acc);
+    return;
+  }
+  auto get = [&](int, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
+    oa = typename C::Operand{a.G, a.ldg, m0, a.M, a.K};
+    ob = typename C::Operand{a.W, a.ldw, n0, a.N, a.K};
+    kb = k_begin;
+    ke = k_end;
+  };
+  auto epilogue = [&](int, float16v (&acc)[C::FM][C::FN]) { store(acc); };
+  C::run(0, 1, lds, get, epilogue);
 }
 
 // out[m][n] = alpha * sum_s part[s][m][n] + beta * out[m][n]; one thread per 4 columns.
@@ -264,10 +302,10 @@ __global__ void __launch_bounds__(256) dx_reduce_kernel(const float* __restrict_
 // ---------------------------------------------------------------------------------------------
 enum DwMode { DW_OUT = 0, DW_UPDATE = 1 };
 
-using DwCore = GemmCore<128, 256, 64, 2, 2, false, false>;
-constexpr int DW_STAGE_PITCH = 72;  // floats per staged row (64 + 8: rows 4 apart land 32 banks apart)
-constexpr int DW_STAGE_BYTES = 4 * 32 * DW_STAGE_PITCH * 4;
-constexpr int DW_LDS_BYTES = DwCore::STAGE_HALVES * 2 > DW_STAGE_BYTES ? DwCore::STAGE_HALVES * 2 : DW_STAGE_BYTES;
+using DwCore = PipeCore<128, 256, 32, 2, 2, 3, false, false, 0>;
+constexpr int DW_STAGE_FLOATS = 8 * 64;  // per wave: 8 label rows x 64 dims
+constexpr int DW_LDS_BYTES = DwCore::LDS_BYTES + DwCore::NW * DW_STAGE_FLOATS * 4;
+static_assert(DwCore::FN % 2 == 0, "epilogue walks pairs of 32-column blocks");
 
 struct DwArgs {
   const half_t* G; int64_t ldg;   // K x M (batch rows x labels), label-contiguous
@@ -279,88 +317,94 @@ struct DwArgs {
   // DW_UPDATE
   half_t* Wt; int64_t ldw; half_t* Mo; int64_t ldm; float lr, mu, wd;
   float* dw_dump; int64_t ld_dump;  // optional copy of dW (may be null)
-  int tiles_m, tiles_n;
+  int tiles_m, tiles_n, n_ids;      // n_ids = tiles_n * round_up(tiles_m, 8)
 };
 
+// Persistent, two workgroups per CU: workgroup w takes tile ids w, w + gridDim.x, ...; the dim tiles of
+// one label tile have neighbouring ids on one XCD, so its slice of G is fetched from HBM once.
 template <int MODE>
 __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
   using C = DwCore;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
-  int nt, mt;
-  xcd_map(blockIdx.x, a.tiles_n, nt, mt);
-  if (mt >= a.tiles_m) return;
-  const int m0 = mt * C::BM, n0 = nt * C::BN;
-  float16v acc[C::FM][C::FN];
-#pragma unroll
-  for (int i = 0; i < C::FM; ++i)
-#pragma unroll
-    for (int j = 0; j < C::FN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  typename C::Operand oa{a.G, a.ldg, m0, a.g_cols, a.K};
-  typename C::Operand ob{a.X, a.ldx, n0, a.N, a.K};
-  C::template run<1>(oa, ob, 0, a.K, lds, acc);
-
+  const int G = gridDim.x, w = blockIdx.x;
+  const int n_items = (a.n_ids - w + G - 1) / G;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
-  float* stage = reinterpret_cast<float*>(smem_raw) + wave * 32 * DW_STAGE_PITCH;
+  float* stage = reinterpret_cast<float*>(smem_raw + C::LDS_BYTES) + wave * DW_STAGE_FLOATS;
+
+  auto get = [&](int item, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
+    int nt, mt;
+    xcd_map(item * G + w, a.tiles_n, nt, mt);
+    oa = typename C::Operand{a.G, a.ldg, mt * C::BM, mt < a.tiles_m ? a.g_cols : 0, a.K};
+    ob = typename C::Operand{a.X, a.ldx, nt * C::BN, a.N, a.K};
+    kb = 0;
+    ke = a.K;
+  };
+  auto epilogue = [&](int item, float16v (&acc)[C::FM][C::FN]) {
+    int nt, mt;
+    xcd_map(item * G + w, a.tiles_n, nt, mt);
+    if (mt >= a.tiles_m) return;
+    const int m0 = mt * C::BM, n0 = nt * C::BN;
+    const int h = lane >> 5;
+    const int srow = lane >> 3, sch = lane & 7;  // staging read: 8 rows x 8 chunks of 8 dims
 #pragma unroll
-  for (int fm = 0; fm < C::FM; ++fm) {
+    for (int fm = 0; fm < C::FM; ++fm) {
 #pragma unroll
-    for (int fp = 0; fp < C::FN / 2; ++fp) {
-      __syncthreads();
+      for (int q = 0; q < 4; ++q) {
 #pragma unroll
-      for (int q = 0; q < 2; ++q)
+        for (int fp = 0; fp < C::FN / 2; ++fp) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          stage[c_row(r, lane) * DW_STAGE_PITCH + 32 * q + (lane & 31)] = acc[fm][2 * fp + q][r];
-      __syncthreads();
+          for (int f = 0; f < 2; ++f)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int cid = lane + 64 * i;
-        const int lr = cid >> 3, ch = cid & 7;
-        const int row = m0 + wm * C::TM + fm * 32 + lr;
-        const int col = n0 + wn * C::TN + fp * 64 + ch * 8;
-        if (row >= a.M || col >= a.N) continue;
-        const float4v v0 = *reinterpret_cast<const float4v*>(stage + lr * DW_STAGE_PITCH + ch * 8);
-        const float4v v1 = *reinterpret_cast<const float4v*>(stage + lr * DW_STAGE_PITCH + ch * 8 + 4);
-        float g[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        if constexpr (MODE == DW_OUT) {
-          float* o = a.out + (int64_t)row * a.ldo + col;
-          float4v o0, o1;
+            for (int rr = 0; rr < 4; ++rr)
+              stage[(4 * h + rr) * 64 + f * 32 + (lane & 31)] = acc[fm][2 * fp + f][4 * q + rr];
+          // the wave's own LDS traffic is ordered: the writes above are visible to the reads below
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          const float4v v0 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8);
+          const float4v v1 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8 + 4);
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
+          const int col = n0 + wn * C::TN + fp * 64 + sch * 8;
+          if (row >= a.M || col >= a.N) continue;
+          const float g[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+          if constexpr (MODE == DW_OUT) {
+            float* o = a.out + (int64_t)row * a.ldo + col;
+            float4v o0, o1;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
-          if (a.beta != 0.f) {
-            o0 += a.beta * *reinterpret_cast<const float4v*>(o);
-            o1 += a.beta * *reinterpret_cast<const float4v*>(o + 4);
+            for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
+            if (a.beta != 0.f) {
+              o0 += a.beta * *reinterpret_cast<const float4v*>(o);
+              o1 += a.beta * *reinterpret_cast<const float4v*>(o + 4);
+            }
+            *reinterpret_cast<float4v*>(o) = o0;
+            *reinterpret_cast<float4v*>(o + 4) = o1;
+          } else {
+            half_t* wp = a.Wt + (int64_t)row * a.ldw + col;
+            half_t* mp = a.Mo + (int64_t)row * a.ldm + col;
+            half8 wv = *reinterpret_cast<const half8*>(wp);
+            half8 mv = *reinterpret_cast<const half8*>(mp);
+            if (a.dw_dump) {
+              float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
+              *reinterpret_cast<float4v*>(d) = v0;
+              *reinterpret_cast<float4v*>(d + 4) = v1;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float wf = (float)wv[e];
+              const float gg = g[e] + a.wd * wf;
+              const float mf = a.mu * (float)mv[e] + gg;
+              mv[e] = (half_t)mf;
+              wv[e] = (half_t)(wf - a.lr * mf);
+            }
+            *reinterpret_cast<half8*>(mp) = mv;
+            *reinterpret_cast<half8*>(wp) = wv;
           }
-          *reinterpret_cast<float4v*>(o) = o0;
-          *reinterpret_cast<float4v*>(o + 4) = o1;
-        } else {
-          half_t* wp = a.Wt + (int64_t)row * a.ldw + col;
-          half_t* mp = a.Mo + (int64_t)row * a.ldm + col;
-          half8 w = *reinterpret_cast<const half8*>(wp);
-          half8 m = *reinterpret_cast<const half8*>(mp);
-          if (a.dw_dump) {
-            float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
-            *reinterpret_cast<float4v*>(d) = v0;
-            *reinterpret_cast<float4v*>(d + 4) = v1;
-          }
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float wf = (float)w[e];
-            const float gg = g[e] + a.wd * wf;
-            const float mf = a.mu * (float)m[e] + gg;
-            m[e] = (half_t)mf;
-            w[e] = (half_t)(wf - a.lr * mf);
-          }
-          *reinterpret_cast<half8*>(mp) = m;
-          *reinterpret_cast<half8*>(wp) = w;
         }
       }
     }
-  }
+  };
+  C::run(0, n_items, lds, get, epilogue);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -434,6 +478,17 @@ int check_launch() {
   return XFC_OK;
 }
 
+// Launch with `lds` bytes of dynamic LDS; sizes above the default limit need the attribute once per kernel.
+template <class K, class A>
+void launch_k(K kernel, dim3 g, dim3 b, int lds, hipStream_t st, const A& args) {
+  static bool raised = false;
+  if (!raised && lds > 48 * 1024) {
+    hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, g, b, lds, st, args);
+}
+
 int num_cus() {
   static int n = 0;
   if (n == 0) {
@@ -476,23 +531,27 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   a.ent_col = bk ? bk->ent_col : nullptr;
   a.tiles_m = ceil_div(M, FwdCore::BM);
   a.tiles_n = ceil_div(n_store, FwdCore::BN);
-  const int64_t grid = (int64_t)a.tiles_m * round_up(a.tiles_n, 8);
-  if (grid <= 0) return XFC_OK;
-  if (grid > 0x7fffffff) return XFC_ERR_INVALID;
-  dim3 g((unsigned)grid), b(256);
-  if (mode == FWD_GRAD) hipLaunchKernelGGL(fwd_kernel<FWD_GRAD>, g, b, FWD_LDS_BYTES, st, a);
-  else if (mode == FWD_SIGMOID) hipLaunchKernelGGL(fwd_kernel<FWD_SIGMOID>, g, b, FWD_LDS_BYTES, st, a);
-  else hipLaunchKernelGGL(fwd_kernel<FWD_LINEAR>, g, b, FWD_LDS_BYTES, st, a);
+  const int64_t ids = (int64_t)a.tiles_m * round_up(a.tiles_n, 8);
+  if (ids <= 0) return XFC_OK;
+  if (ids > 0x7fffffff) return XFC_ERR_INVALID;
+  a.n_ids = (int)ids;
+  int64_t grid = (int64_t)round_up(num_cus(), 8);  // one resident workgroup per CU
+  if (grid > ids) grid = ids;                    // ids is a multiple of 8
+  dim3 g((unsigned)grid), b(FwdCore::NT);
+  if (mode == FWD_GRAD) launch_k(fwd_kernel<FWD_GRAD, false>, g, b, FWD_LDS_BYTES, st, a);
+  else if (mode == FWD_SIGMOID && beta != 0.f) launch_k(fwd_kernel<FWD_SIGMOID, true>, g, b, FWD_LDS_BYTES, st, a);
+  else if (mode == FWD_SIGMOID) launch_k(fwd_kernel<FWD_SIGMOID, false>, g, b, FWD_LDS_BYTES, st, a);
+  else launch_k(fwd_kernel<FWD_LINEAR, false>, g, b, FWD_LDS_BYTES, st, a);
   return check_launch();
 }
 
-// Split count for dX: enough workgroups for two per CU, a multiple of 8 (one slice of the
-// label axis per XCD at a time), each slice a multiple of the k-step.
+// Split count for dX: one workgroup per CU, a multiple of 8 slices (one slice of the label axis per
+// XCD at a time), each slice a multiple of the k-step.
 void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& k_per_split) {
   tiles_m = ceil_div(M, DxCore::BM);
   tiles_n = ceil_div(N, DxCore::BN);
   const int tiles = tiles_m * tiles_n;
-  int s = (2 * num_cus()) / (tiles > 0 ? tiles : 1);
+  int s = num_cus() / (tiles > 0 ? tiles : 1);
   s = s / 8 * 8;
   if (s < 8) s = 8;
   const int max_s = (int)round_up(ceil_div(K, DxCore::BK), 8);
@@ -511,7 +570,7 @@ int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float*
   a.M = M; a.N = N; a.K = K;
   const int64_t grid = (int64_t)a.tiles_m * a.tiles_n * a.splits;
   if (grid <= 0 || M <= 0 || N <= 0) return XFC_OK;
-  hipLaunchKernelGGL(dx_kernel, dim3((unsigned)grid), dim3(256), DX_LDS_BYTES, st, a);
+  launch_k(dx_kernel, dim3((unsigned)grid), dim3(DxCore::NT), DX_LDS_BYTES, st, a);
   int rc = check_launch();
   if (rc) return rc;
   const int64_t nq = (int64_t)M * (N / 4);
@@ -523,13 +582,14 @@ int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float*
 int launch_dw(int mode, DwArgs a, hipStream_t st) {
   a.tiles_m = ceil_div(a.M, DwCore::BM);
   a.tiles_n = ceil_div(a.N, DwCore::BN);
-  const int64_t grid = (int64_t)a.tiles_n * round_up(a.tiles_m, 8);
-  if (grid <= 0) return XFC_OK;
-  if (grid > 0x7fffffff) return XFC_ERR_INVALID;
-  if (mode == DW_UPDATE)
-    hipLaunchKernelGGL(dw_kernel<DW_UPDATE>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
-  else
-    hipLaunchKernelGGL(dw_kernel<DW_OUT>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  const int64_t ids = (int64_t)a.tiles_n * round_up(a.tiles_m, 8);
+  if (ids <= 0) return XFC_OK;
+  if (ids > 0x7fffffff) return XFC_ERR_INVALID;
+  a.n_ids = (int)ids;
+  int64_t grid = 2 * (int64_t)round_up(num_cus(), 8);  // two resident workgroups per CU
+  if (grid > ids) grid = ids / 8 * 8 > 0 ? ids / 8 * 8 : ids;
+  if (mode == DW_UPDATE) launch_k(dw_kernel<DW_UPDATE>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  else launch_k(dw_kernel<DW_OUT>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
   return check_launch();
 }
 
@@ -586,8 +646,8 @@ int xfc_gemm(const void* in1, int64_t in1_rows, int64_t in1_cols, int64_t in1_s0
   if (apply_sigmoid) {
     // out(fp16) = sigmoid(alpha * in1 . in2 + beta * out), in1 row-major, in2 column-major
     if (!(a_row && b_col)) return XFC_ERR_LAYOUT;
-    const bool fast = out_s1 == 1 && in1_s0 % 8 == 0 && in2_s1 % 8 == 0 && K % 8 == 0 && aligned16(in1) &&
-                      aligned16(in2) && K > 0;
+    const bool fast = out_s1 == 1 && out_s0 % 8 == 0 && aligned16(out) && in1_s0 % 8 == 0 && in2_s1 % 8 == 0 &&
+                      K % 8 == 0 && aligned16(in1) && aligned16(in2) && K > 0;
     if (fast)
       return launch_fwd(FWD_SIGMOID, (const half_t*)in1, in1_s0, (const half_t*)in2, in2_s1, (half_t*)out, out_s0,
                         (int)M, (int)N, (int)K, (int)N, alpha, beta, nullptr, st);
@@ -627,7 +687,9 @@ int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out
   if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
   if (B == 0 || L == 0) return XFC_OK;
   if (!X || !W || !out || d <= 0) return XFC_ERR_INVALID;
-  if (ldx % 8 || ldw % 8 || d % 8 || !aligned16(X) || !aligned16(W)) return XFC_ERR_ALIGN;
+  if (ldx % 8 || ldw % 8 || ldo % 8 || d % 8 || !aligned16(X) || !aligned16(W) || !aligned16(out))
+    return XFC_ERR_ALIGN;
+  if (ldo < L) return XFC_ERR_SHAPE;
   return launch_fwd(FWD_LINEAR, (const half_t*)X, ldx, (const half_t*)W, ldw, (half_t*)out, ldo, (int)B, (int)L, (int)d,
                     (int)L, 1.0f, 0.0f, nullptr, reinterpret_cast<hipStream_t>(stream));
 }
@@ -644,7 +706,8 @@ static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw,
   if (B == 0 || L == 0) return XFC_OK;
   if (!X || !W || !G || d <= 0) return XFC_ERR_INVALID;
   if (nnz > 0 && !((rowptr && colidx) || (pos_x && pos_y))) return XFC_ERR_INVALID;
-  if (ldx % 8 || ldw % 8 || d % 8 || !aligned16(X) || !aligned16(W)) return XFC_ERR_ALIGN;
+  if (ldx % 8 || ldw % 8 || ldg % 8 || d % 8 || !aligned16(X) || !aligned16(W) || !aligned16(G))
+    return XFC_ERR_ALIGN;
   if (ldg < L) return XFC_ERR_SHAPE;
   if (!ws || ws_bytes < bucket_ws_bytes(L, nnz)) return XFC_ERR_WORKSPACE;
   BucketWs bk = carve_bucket_ws(ws, L, nnz);
@@ -655,9 +718,9 @@ static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw,
                      FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
   int rc = check_launch();
   if (rc) return rc;
-  // label columns L .. min(ldg, round_up(L, 8)) are written as zero so that G can be read in
-  // 16-byte pieces along the label axis by the dX and dW kernels
-  const int64_t n_store = round_up(L, 8) <= ldg ? round_up(L, 8) : L;
+  // label columns L .. round_up(L, 8) are written as zero so that G can be read in 16-byte
+  // pieces along the label axis by the dX and dW kernels (ldg is a multiple of 8, so they exist)
+  const int64_t n_store = round_up(L, 8);
   return launch_fwd(FWD_GRAD, (const half_t*)X, ldx, (const half_t*)W, ldw, (half_t*)G, ldg, (int)B, (int)L, (int)d,
                     (int)n_store, 1.0f, 0.0f, &bk, st);
 }
