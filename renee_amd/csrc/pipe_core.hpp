@@ -76,7 +76,7 @@ __device__ __forceinline__ int kc_swz(int row) {
 // transposing read touches then sit in four different 64-byte bank groups.
 __device__ __forceinline__ int mc_swz(int k) { return (k & 3) << 2; }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_, int PF_ = 3>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_>
 struct PipeCore {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
@@ -86,107 +86,94 @@ struct PipeCore {
   static constexpr int CPR = BK / 8;
   static constexpr int A_HALVES = BM * BK, B_HALVES = BN * BK;
   static constexpr int STAGE_HALVES = A_HALVES + B_HALVES;
-  static constexpr int RING_BYTES = STAGES * STAGE_HALVES * 2;
-  static constexpr int LDS_BYTES = RING_BYTES + (PF_ > 0 ? WM * WN * 256 : 0);
+  static constexpr int LDS_BYTES = STAGES * STAGE_HALVES * 2;
   static constexpr int A_CH = BM * BK / 8 / NT, B_CH = BN * BK / 8 / NT;
-  static constexpr int PF = PF_;  // the L2 is warmed this many stages ahead of the LDS fill (0: off)
-  static constexpr int LOADS_PER_STAGE = A_CH + B_CH + (PF > 0 ? 1 : 0);
+  static constexpr int LOADS_PER_STAGE = A_CH + B_CH;
   static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile must be 32-multiples");
   static_assert((BM * BK / 8) % NT == 0 && (BN * BK / 8) % NT == 0, "chunk split");
   static_assert(BK == 32 || BK == 64, "BK");
   static_assert(A_KC || BM >= 128, "MC swizzle needs 16 chunks per k-row");
   static_assert(B_KC || BN >= 128, "MC swizzle needs 16 chunks per k-row");
   static_assert(STAGES >= 2 && (STAGES - 1) * LOADS_PER_STAGE < 64, "stages");
+  static_assert(NW % 2 == 0, "the LDS swizzles assume an even number of waves");
 
+  // One operand's tile: base pointer, leading dimension (halves), first row (KC) or column (MC) of the
+  // tile, the limit of that index and the limit of the contraction index.  Requirements: r0 < rmax;
+  // for MC operands rmax is a multiple of 8; ld * 2 * 16 < 2^32.  Rows (columns) at or past rmax are
+  // fetched from the last valid row (column chunk) instead: they only ever feed outputs the caller
+  // discards.  Contraction indices at or past kmax are fetched as zeros.
   struct Operand {
     const half_t* p;
     int64_t ld;
-    int r0, rmax, kmax;  // first row (or column) of the tile, its limit, limit of the k index
+    int r0, rmax, kmax;
   };
 
-  // Per-thread addresses of the CH 16-byte pieces it fetches for one operand each stage.
+  // Addresses of the CH 16-byte pieces a thread fetches for one operand each stage.  Every fetch is
+  // "uniform 64-bit base + per-thread 32-bit offset": the bases advance along k with scalar adds, so a
+  // steady-state stage costs no vector ALU work, which matters because the SIMD that issues the MFMAs
+  // cannot overlap them with other vector instructions.
   template <bool KC, int R, int CH>
   struct Loader {
-    const half_t* ptr[CH];
-    int koff[CH];
-    uint32_t ok;
-    int kmax;
-    int64_t kstride;
+    static constexpr int CPI = KC ? CPR : R / 8;  // 16-byte chunks per tile row (KC) or per k-row (MC)
+    static constexpr int RPI = 64 / CPI;          // tile rows (KC) or k-rows (MC) one wave instruction covers
+    const char* base;    // uniform
+    int64_t grp[CH];     // uniform byte offset of each instruction's first row
+    uint32_t voff[CH];   // per-thread byte offset inside the group
+    int64_t kbytes;      // uniform byte offset of the current stage along k
+    int64_t kstep;       // uniform
+    int kmax, kin;       // limit of k; per-thread k offset inside the stage (KC: chunk*8, MC: k-row in group)
+    int kgrp[CH];        // uniform: first k-row of each instruction (MC), 0 (KC)
     __device__ __forceinline__ void init(const Operand& o, int k_begin, int wave, int lane) {
-      ok = 0u;
+      base = reinterpret_cast<const char*>(o.p);
       kmax = o.kmax;
-      kstride = KC ? (int64_t)BK : (int64_t)BK * o.ld;
+      const int sub = lane / CPI, pc = lane % CPI;
+      if constexpr (KC) {
+        kstep = (int64_t)BK * 2;
+        kbytes = (int64_t)k_begin * 2;
+        const int c = pc ^ kc_swz<BK>(wave * RPI + sub);  // the swizzle does not depend on i (NW is even)
+        kin = c * 8;
 #pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const int q = (i * NW + wave) * 64 + lane;
-        int r, k;
-        if constexpr (KC) {
-          const int row = q / CPR, pc = q % CPR;
-          r = row;
-          k = (pc ^ kc_swz<BK>(row)) * 8;
-        } else {
-          const int krow = q / (R / 8), pc = q % (R / 8);
-          k = krow;
-          r = (pc ^ mc_swz(krow)) * 8;
+        for (int i = 0; i < CH; ++i) {
+          const int row0 = o.r0 + (i * NW + wave) * RPI;
+          const int g = row0 < o.rmax ? row0 : o.rmax - 1;
+          const int row = row0 + sub < o.rmax ? row0 + sub : o.rmax - 1;
+          grp[i] = (int64_t)g * o.ld * 2;
+          voff[i] = (uint32_t)(row - g) * (uint32_t)(o.ld * 2) + (uint32_t)c * 16u;
+          kgrp[i] = 0;
         }
-        const int gr = o.r0 + r;
-        if (gr < o.rmax) ok |= 1u << i;
-        koff[i] = k;
-        const int gk = k_begin + k;
-        ptr[i] = KC ? o.p + (int64_t)gr * o.ld + gk : o.p + (int64_t)gk * o.ld + gr;
+      } else {
+        kstep = (int64_t)BK * o.ld * 2;
+        kbytes = (int64_t)k_begin * o.ld * 2;
+        const int c = pc ^ mc_swz(wave * RPI + sub);
+        const int col = o.r0 + c * 8 < o.rmax ? o.r0 + c * 8 : o.rmax - 8;
+        kin = sub;
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+          kgrp[i] = (i * NW + wave) * RPI;
+          grp[i] = (int64_t)kgrp[i] * o.ld * 2;
+          voff[i] = (uint32_t)sub * (uint32_t)(o.ld * 2) + (uint32_t)col * 2u;
+        }
       }
     }
     // k0: absolute k of the stage being fetched
     __device__ __forceinline__ void issue(half_t* region, int k0, int wave) {
+      if (k0 + BK <= kmax) {
 #pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const bool valid = ((ok >> i) & 1u) && (k0 + koff[i] < kmax);
-        const void* src = valid ? (const void*)ptr[i] : (const void*)g_zero16;
-        load16_to_lds(src, region + (i * NW + wave) * 512);
-        ptr[i] += kstride;
+        for (int i = 0; i < CH; ++i)
+          load16_to_lds(base + grp[i] + kbytes + voff[i], region + (i * NW + wave) * 512);
+      } else {  // the stage that crosses kmax: pieces past it come from the block of zeros
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+          const bool valid = k0 + kgrp[i] + kin < kmax;
+          const void* src = valid ? (const void*)(base + grp[i] + kbytes + voff[i]) : (const void*)g_zero16;
+          load16_to_lds(src, region + (i * NW + wave) * 512);
+        }
       }
+      kbytes += kstep;
     }
   };
   using LoaderA = Loader<A_KC, BM, A_CH>;
   using LoaderB = Loader<B_KC, BN, B_CH>;
-
-  // L2 warm-up: HBM latency (microseconds under load) is longer than the ring can cover, so every
-  // thread touches one 128-byte line of a stage PF stages before that stage's LDS fill is issued
-  // (4 bytes per lane into a scratch corner of LDS).  The first half of the workgroup's threads
-  // walks operand A's lines, the second half operand B's; the fill then finds its data in L2.
-  struct Prefetcher {
-    const half_t* ptr;
-    int koff, kmax;
-    bool ok;
-    int64_t kstride;
-    template <bool KC, int R>
-    __device__ __forceinline__ void init_op(const Operand& o, int k_begin, int u) {
-      kmax = o.kmax;
-      kstride = KC ? (int64_t)BK : (int64_t)BK * o.ld;
-      if constexpr (KC) {
-        const int row = u;  // one line per row when BK == 64 (half a line when 32)
-        ok = u < R && o.r0 + row < o.rmax;
-        koff = 0;
-        ptr = o.p + (int64_t)(o.r0 + row) * o.ld + k_begin;
-      } else {
-        constexpr int LPR = R / 64;  // 128-byte lines per k-row
-        const int krow = u / LPR, seg = u % LPR;
-        ok = u < BK * LPR && o.r0 + seg * 64 < o.rmax;
-        koff = krow;
-        ptr = o.p + (int64_t)(k_begin + krow) * o.ld + o.r0 + seg * 64;
-      }
-    }
-    __device__ __forceinline__ void init(const Operand& oa, const Operand& ob, int k_begin) {
-      const int t = threadIdx.x;
-      if (t < NT / 2) init_op<A_KC, BM>(oa, k_begin, t);
-      else init_op<B_KC, BN>(ob, k_begin, t - NT / 2);
-    }
-    __device__ __forceinline__ void issue(void* lds_scratch, int k0) {
-      const void* src = (ok && k0 + koff < kmax) ? (const void*)ptr : (const void*)g_zero16;
-      __builtin_amdgcn_global_load_lds((XFC_GLB const void*)src, (XFC_LDS void*)lds_scratch, 4, 0, 0);
-      ptr += kstride;
-    }
-  };
 
   __device__ __forceinline__ static half8 frag_kc(const half_t* lds, int row0, int kk, int lane) {
     const int r = row0 + (lane & 31);
@@ -267,37 +254,6 @@ struct PipeCore {
     float16v acc[FM][FN];
     zero(acc);
 
-    // warm-up cursor: PF stages ahead of the fill cursor
-    Prefetcher pf;
-    int p_item = item_begin, p_k = 0, p_kend = 0;
-    bool p_live = PF > 0;
-    void* pf_lds = reinterpret_cast<unsigned char*>(lds) + RING_BYTES + wave * 256;
-    if constexpr (PF > 0) {
-      Operand oa, ob;
-      get(p_item, oa, ob, p_k, p_kend);
-      pf.init(oa, ob, p_k);
-    }
-    auto prefetch_one = [&]() {
-      if constexpr (PF > 0) {
-        if (p_live) {
-          pf.issue(pf_lds, p_k);
-          p_k += BK;
-          if (p_k >= p_kend) {
-            ++p_item;
-            if (p_item < item_end) {
-              Operand oa, ob;
-              get(p_item, oa, ob, p_k, p_kend);
-              pf.init(oa, ob, p_k);
-            } else {
-              p_live = false;
-            }
-          }
-        } else {
-          __builtin_amdgcn_global_load_lds((XFC_GLB const void*)g_zero16, (XFC_LDS void*)pf_lds, 4, 0, 0);
-        }
-      }
-    };
-
     // fill cursor
     LoaderA la;
     LoaderB lb;
@@ -329,15 +285,10 @@ struct PipeCore {
       } else {
         // past the last stage: keep the count of outstanding fetches per iteration constant
 #pragma unroll
-        for (int i = 0; i < A_CH + B_CH; ++i) load16_to_lds((const void*)g_zero16, st + (i * NW + wave) * 512);
+        for (int i = 0; i < LOADS_PER_STAGE; ++i) load16_to_lds((const void*)g_zero16, st + (i * NW + wave) * 512);
       }
       i_slot = i_slot + 1 == STAGES ? 0 : i_slot + 1;
-      prefetch_one();  // issued after the fill, so the fill is never behind a younger, slower request
     };
-    if constexpr (PF > 0) {
-#pragma unroll
-      for (int s = 0; s < PF; ++s) prefetch_one();
-    }
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) issue_one();
     wait_vmcnt_barrier<(STAGES - 2) * LOADS_PER_STAGE>();

@@ -105,7 +105,7 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
 // ---------------------------------------------------------------------------------------------
 enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2 };
 
-using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true, 0>;
+using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true>;
 constexpr int FWD_AUX_BYTES = FwdCore::BN * (FwdCore::BM / 32) * 4;  // bitmap, then 8 x 64 halves of staging per wave
 static_assert(FWD_AUX_BYTES >= FwdCore::NW * 512 * 2 && FwdCore::FN == 2, "staging fits the bitmap area");
 constexpr int FWD_LDS_BYTES = FwdCore::LDS_BYTES + FWD_AUX_BYTES;
@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
     int mt, nt;
     xcd_map(item * G + w, a.tiles_m, mt, nt);
     oa = typename C::Operand{a.X, a.ldx, mt * C::BM, a.M, a.K};
-    ob = typename C::Operand{a.W, a.ldw, nt * C::BN, nt < a.tiles_n ? a.N : 0, a.K};
+    ob = typename C::Operand{a.W, a.ldw, nt < a.tiles_n ? nt * C::BN : 0, a.N, a.K};
     kb = 0;
     ke = a.K;
   };
@@ -221,7 +221,7 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
 // ---------------------------------------------------------------------------------------------
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
-using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, 0>;
+using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false>;
 constexpr int DX_LDS_BYTES = DxCore::LDS_BYTES;
 
 struct DxArgs {
@@ -302,7 +302,7 @@ __global__ void __launch_bounds__(256) dx_reduce_kernel(const float* __restrict_
 // ---------------------------------------------------------------------------------------------
 enum DwMode { DW_OUT = 0, DW_UPDATE = 1 };
 
-using DwCore = PipeCore<128, 256, 32, 2, 2, 3, false, false, 0>;
+using DwCore = PipeCore<128, 256, 32, 2, 2, 3, false, false>;
 constexpr int DW_STAGE_FLOATS = 8 * 64;  // per wave: 8 label rows x 64 dims
 constexpr int DW_LDS_BYTES = DwCore::LDS_BYTES + DwCore::NW * DW_STAGE_FLOATS * 4;
 static_assert(DwCore::FN % 2 == 0, "epilogue walks pairs of 32-column blocks");
@@ -336,7 +336,7 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
   auto get = [&](int item, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
     int nt, mt;
     xcd_map(item * G + w, a.tiles_n, nt, mt);
-    oa = typename C::Operand{a.G, a.ldg, mt * C::BM, mt < a.tiles_m ? a.g_cols : 0, a.K};
+    oa = typename C::Operand{a.G, a.ldg, mt < a.tiles_m ? mt * C::BM : 0, a.g_cols, a.K};
     ob = typename C::Operand{a.X, a.ldx, nt * C::BN, a.N, a.K};
     kb = 0;
     ke = a.K;
