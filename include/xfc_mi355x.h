@@ -145,6 +145,23 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* M, int6
                  float lr, float momentum, float weight_decay, float scale,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Exact top-K labels per query row over all L labels, logits never written:
+ *   values[b][0..K-1], indices[b][0..K-1] = the K largest X[b].W[l], ties broken towards
+ *   the lower label id.
+ * Replaces FullPredictor's scoring loop, dl_base.py:736-756 (xfc_forward into outsoft,
+ * then torch.max K times with the winners overwritten) and the pad clamp at
+ * dl_base.py:782: indices >= numy are returned as numy-1.  1 <= K <= 8 <= L (the
+ * reference's K > 5 branch, torch.topk at :756, is served by xfc_logits + a sort).
+ * values are the fp32 accumulators (the reference returns the fp16-rounded logits).
+ * Workspace: xfc_topk_workspace_bytes(B, L, K) bytes.
+ */
+size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K);
+int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw,
+             int64_t B, int64_t L, int64_t d, int64_t numy, int K,
+             float* values, int64_t* indices,
+             void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

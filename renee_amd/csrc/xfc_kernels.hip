@@ -219,6 +219,202 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// top-K labels per row of X . W^T, never writing the logits (K <= 8)
+// ---------------------------------------------------------------------------------------------
+// Each workgroup owns 256 query rows and walks every n_groups-th label tile with the forward main loop.
+// Per row it keeps the K best (score, label) pairs seen so far, ordered by score descending and label
+// ascending (the order iterated torch.max produces: first maximum wins ties).  A finished tile is first
+// filtered against each row's current K-th score; survivors (few once the lists have warmed up) go to
+// a small per-row buffer that the row's owner thread merges.  If any row overflows its buffer, the tile
+// is rescanned exactly, eight columns at a time.  A second kernel merges the groups' lists.
+constexpr int TOPK_MAX = 8;
+constexpr int TOPK_CAP = 4;  // filtered candidates a row can take per tile on the fast path
+using TopkCore = FwdCore;
+struct TopkLds {
+  float list_v[TopkCore::BM][TOPK_MAX];
+  int32_t list_i[TopkCore::BM][TOPK_MAX];
+  float tau[TopkCore::BM];
+  int32_t cnt[TopkCore::BM];
+  float buf_v[TopkCore::BM][TOPK_CAP];  // fast path: candidates; slow path: 8 staged columns (with buf_i)
+  int32_t buf_i[TopkCore::BM][TOPK_CAP];
+  int32_t overflow;
+};
+constexpr int TOPK_LDS_BYTES = TopkCore::LDS_BYTES + (int)sizeof(TopkLds);
+static_assert(TOPK_LDS_BYTES <= 160 * 1024, "top-K LDS budget");
+static_assert(2 * TOPK_CAP == 8, "the exact rescan stages 8 columns in the candidate buffers");
+
+struct TopkArgs {
+  const half_t* X; int64_t ldx;
+  const half_t* W; int64_t ldw;
+  int M, N, K;          // rows, labels, feature dims
+  int topk;
+  float* cand_v; int32_t* cand_i;  // [n_groups][M][topk]
+  int tiles_m, tiles_n, n_groups;
+};
+
+__device__ __forceinline__ bool topk_better(float av, int ai, float bv, int bi) {
+  return av > bv || (av == bv && ai < bi);
+}
+__device__ __forceinline__ void topk_insert(float* lv, int32_t* li, int K, float v, int i) {
+  if (!topk_better(v, i, lv[K - 1], li[K - 1])) return;
+  int p = K - 1;
+  while (p > 0 && topk_better(v, i, lv[p - 1], li[p - 1])) {
+    lv[p] = lv[p - 1];
+    li[p] = li[p - 1];
+    --p;
+  }
+  lv[p] = v;
+  li[p] = i;
+}
+
+// Out of line on purpose: inlined 128 times into the filter, the compiler merges the bodies and the
+// register pressure of the whole epilogue explodes.
+__device__ __attribute__((noinline)) void topk_push(TopkLds& S, int row, float v, int col) {
+  const int slot = atomicAdd(&S.cnt[row], 1);
+  if (slot < TOPK_CAP) { S.buf_v[row][slot] = v; S.buf_i[row][slot] = col; }
+  else S.overflow = 1;
+}
+
+__global__ void __launch_bounds__(TopkCore::NT) topk_kernel(TopkArgs a) {
+  using C = TopkCore;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  half_t* lds = reinterpret_cast<half_t*>(smem_raw);
+  TopkLds& S = *reinterpret_cast<TopkLds*>(smem_raw + C::LDS_BYTES);
+  // ids are dealt round-robin to XCDs: the row tiles of one label group sit side by side on one XCD
+  int mt, grp;
+  xcd_map(blockIdx.x, a.tiles_m, mt, grp);
+  const int n_items = grp < a.tiles_n ? (a.tiles_n - grp + a.n_groups - 1) / a.n_groups : 0;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / C::WN, wn = wave % C::WN;
+  const int m0 = mt * C::BM;
+  const int K = a.topk;
+  const float NEG_INF = -__builtin_huge_valf();
+  for (int t = threadIdx.x; t < C::BM; t += C::NT) {
+    for (int j = 0; j < TOPK_MAX; ++j) { S.list_v[t][j] = NEG_INF; S.list_i[t][j] = 0x7fffffff; }
+    S.tau[t] = NEG_INF;
+    S.cnt[t] = 0;
+  }
+  if (threadIdx.x == 0) S.overflow = 0;
+  __syncthreads();
+
+  auto get = [&](int item, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
+    const int nt = grp + item * a.n_groups;
+    oa = typename C::Operand{a.X, a.ldx, m0, a.M, a.K};
+    ob = typename C::Operand{a.W, a.ldw, nt * C::BN, a.N, a.K};
+    kb = 0;
+    ke = a.K;
+  };
+  auto epilogue = [&](int item, float16v (&acc)[C::FM][C::FN]) {
+    const int nt = grp + item * a.n_groups;
+    const int n0 = nt * C::BN;
+    const bool ragged = n0 + C::BN > a.N;
+    const int h = lane >> 5;
+    // filter against each row's K-th best so far
+#pragma unroll
+    for (int fm = 0; fm < C::FM; ++fm) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row0 = wm * C::TM + fm * 32 + 8 * q + 4 * h;
+        const float4v tau4 = *reinterpret_cast<const float4v*>(&S.tau[row0]);
+#pragma unroll
+        for (int fn = 0; fn < C::FN; ++fn) {
+          const int col = n0 + wn * C::TN + fn * 32 + (lane & 31);
+          const bool col_ok = !ragged || col < a.N;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const float v = acc[fm][fn][4 * q + rr];
+            if (v > tau4[rr] && col_ok) topk_push(S, row0 + rr, v, col);  // rare once the lists have warmed up
+          }
+        }
+        asm volatile("" ::: "memory");  // keep the threshold reads of later strips from being hoisted up here
+      }
+    }
+    __syncthreads();
+    const bool overflow = S.overflow != 0;
+    if (!overflow) {
+      if (threadIdx.x < C::BM) {
+        const int t = threadIdx.x;
+        const int n = S.cnt[t];
+        for (int i = 0; i < n; ++i) topk_insert(S.list_v[t], S.list_i[t], K, S.buf_v[t][i], S.buf_i[t][i]);
+        if (n) { S.tau[t] = S.list_v[t][K - 1]; S.cnt[t] = 0; }
+      }
+    } else {
+      // exact rescan: stage 8 columns of all 256 rows at a time, each row's owner inserts them
+      float* stage = &S.buf_v[0][0];  // 256 x 8 floats: buf_v and buf_i are adjacent
+      __syncthreads();
+#pragma unroll
+      for (int swn = 0; swn < C::WN; ++swn) {
+#pragma unroll
+        for (int sfn = 0; sfn < C::FN; ++sfn) {
+          for (int sg = 0; sg < 4; ++sg) {
+            if (wn == swn && ((lane & 31) >> 3) == sg) {
+#pragma unroll
+              for (int fm = 0; fm < C::FM; ++fm)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                  stage[(wm * C::TM + fm * 32 + c_row(r, lane)) * 8 + (lane & 7)] = acc[fm][sfn][r];
+            }
+            __syncthreads();
+            if (threadIdx.x < C::BM) {
+              const int t = threadIdx.x;
+              const int cbase = n0 + swn * C::TN + sfn * 32 + sg * 8;
+              for (int e = 0; e < 8; ++e)
+                if (cbase + e < a.N) topk_insert(S.list_v[t], S.list_i[t], K, stage[t * 8 + e], cbase + e);
+            }
+            __syncthreads();
+          }
+        }
+      }
+      if (threadIdx.x < C::BM) { S.tau[threadIdx.x] = S.list_v[threadIdx.x][K - 1]; S.cnt[threadIdx.x] = 0; }
+      if (threadIdx.x == 0) S.overflow = 0;
+    }
+    __syncthreads();
+  };
+  C::run(0, n_items, lds, get, epilogue);
+  __syncthreads();
+  if (threadIdx.x < C::BM && m0 + threadIdx.x < a.M && grp < a.n_groups) {
+    const int64_t o = ((int64_t)grp * a.M + m0 + threadIdx.x) * K;
+    for (int j = 0; j < K; ++j) { a.cand_v[o + j] = S.list_v[threadIdx.x][j]; a.cand_i[o + j] = S.list_i[threadIdx.x][j]; }
+  }
+}
+
+// One wave per row: K rounds of "best pair strictly after the previous pick" over n_groups*K candidates.
+__global__ void __launch_bounds__(64) topk_merge_kernel(const float* __restrict__ cand_v, const int32_t* __restrict__ cand_i,
+                                                        int M, int n_groups, int K, int64_t numy,
+                                                        float* __restrict__ out_v, int64_t* __restrict__ out_i) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const int n = n_groups * K;
+  float pv = __builtin_huge_valf();
+  int pi = -1;
+  for (int r = 0; r < K; ++r) {
+    float bv = -__builtin_huge_valf();
+    int bi = 0x7fffffff;
+    for (int c = lane; c < n; c += 64) {
+      const int g = c / K, j = c % K;
+      const int64_t o = ((int64_t)g * M + row) * K + j;
+      const float v = cand_v[o];
+      const int i = cand_i[o];
+      const bool after_prev = v < pv || (v == pv && i > pi);
+      if (after_prev && topk_better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (topk_better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    pv = bv;
+    pi = bi;
+    if (lane == 0) {
+      out_v[(int64_t)row * K + r] = bv;
+      int64_t idx = bi;
+      if (idx >= numy) idx = numy - 1;  // padded labels are clamped, as the reference does
+      out_i[(int64_t)row * K + r] = idx;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
 using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false>;
@@ -820,6 +1016,49 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int
   rc = xfc_dx(G, ldg, W, ldw, dX, lddx, B, L, d, scale, ws + off, workspace_bytes - off, stream);
   if (rc) return rc;
   return xfc_dw_update(G, ldg, X, ldx, W, ldw, Mo, ldm, B, L, d, lr, momentum, weight_decay, nullptr, 0, stream);
+}
+
+static void topk_plan(int64_t B, int64_t L, int& tiles_m, int& tiles_n, int& n_groups, int& grid) {
+  tiles_m = ceil_div(B, TopkCore::BM);
+  tiles_n = ceil_div(L, TopkCore::BN);
+  int per = num_cus() / (8 * tiles_m);  // groups per XCD
+  if (per < 1) per = 1;
+  n_groups = 8 * per;
+  const int cap = (int)round_up(tiles_n, 8);
+  if (n_groups > cap) n_groups = cap;
+  grid = tiles_m * n_groups;
+}
+
+size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K) {
+  if (!dims_ok(B) || !dims_ok(L) || K < 1 || K > TOPK_MAX || B == 0 || L == 0) return 0;
+  int tm, tn, ng, grid;
+  topk_plan(B, L, tm, tn, ng, grid);
+  return (size_t)ng * B * K * 8;
+}
+
+int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, int64_t L, int64_t d, int64_t numy,
+             int K, float* values, int64_t* indices, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
+  if (B == 0) return XFC_OK;
+  if (K < 1 || K > TOPK_MAX || L < K || numy < 1 || d <= 0) return XFC_ERR_INVALID;
+  if (!X || !W || !values || !indices) return XFC_ERR_INVALID;
+  if (ldx % 8 || ldw % 8 || d % 8 || !aligned16(X) || !aligned16(W)) return XFC_ERR_ALIGN;
+  TopkArgs a;
+  int grid;
+  topk_plan(B, L, a.tiles_m, a.tiles_n, a.n_groups, grid);
+  const size_t need = (size_t)a.n_groups * B * K * 8;
+  if (!workspace || workspace_bytes < need) return XFC_ERR_WORKSPACE;
+  a.X = (const half_t*)X; a.ldx = ldx; a.W = (const half_t*)W; a.ldw = ldw;
+  a.M = (int)B; a.N = (int)L; a.K = (int)d; a.topk = K;
+  a.cand_v = reinterpret_cast<float*>(workspace);
+  a.cand_i = reinterpret_cast<int32_t*>(a.cand_v + (size_t)a.n_groups * B * K);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  launch_k(topk_kernel, dim3((unsigned)grid), dim3(TopkCore::NT), TOPK_LDS_BYTES, st, a);
+  int rc = check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)B), dim3(64), 0, st, a.cand_v, a.cand_i, (int)B, a.n_groups, K,
+                     numy, values, indices);
+  return check_launch();
 }
 
 }  // extern "C"

@@ -146,6 +146,24 @@ class XFCLayer:
         check(rc, "xfc_logits")
         return out
 
+    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None):
+        """Exact top-K labels per row over all labels (FullPredictor's scoring loop, dl_base.py:736-756,
+        with the pad clamp of :782 when numy < the stored label count).  Returns (values fp32, indices
+        int64), each (batch, K); ties go to the lower label id.  K <= 8."""
+        x = self._x16(embed)
+        bsz = x.shape[0]
+        _require(1 <= K <= 8, "K must be in 1..8 (for larger K take xfc_forward and sort)")
+        vals = torch.empty(bsz, K, device=self.device, dtype=torch.float32)
+        inds = torch.empty(bsz, K, device=self.device, dtype=torch.int64)
+        L = lib()
+        with torch.cuda.device(self.device):
+            ws = _workspace.get(self.device, L.xfc_topk_workspace_bytes(bsz, self.numy, K))
+            rc = L.xfc_topk(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims, bsz, self.numy,
+                            self.dims, self.numy if numy is None else int(numy), int(K), vals.data_ptr(),
+                            inds.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))
+        check(rc, "xfc_topk")
+        return vals, inds
+
     def fwd_grad(self, embed, pos_x=None, pos_y=None, rowptr=None, colidx=None) -> torch.Tensor:
         """G = sigmoid(embed . W^T) - Y into outsoft (dl_base.py:591-594); returns the (batch, numy) view."""
         x = self._x16(embed)
