@@ -23,9 +23,9 @@ sys.path.insert(0, ROOT)
 MFMA_F16_PEAK_TFLOPS = 2516.6   # MI355X dense fp16, AMD's published figure
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
-# HBM bytes per launch of the dW+update kernel at configs[2], from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE scaled by a copy kernel of known size (profiles/dw_update_cfg2_pmc.txt); None until measured.
-DW_UPDATE_TRAFFIC_BYTES = {2: None}
+# HBM bytes per launch of the dW+update kernel at configs[2]: rocprofv3 --pmc FETCH_SIZE (2,860,723.5 KiB,
+# x2.000 from the 1 GiB copy) + WRITE_SIZE (3,932,160 KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
+DW_UPDATE_TRAFFIC_BYTES = {2: (2 * 2860723.5 + 3932160.0) * 1024.0}
 
 
 def cpu_baseline(cfg: int, d: int, seed: int):
@@ -71,6 +71,9 @@ def main() -> int:
     ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (1..4)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="after the timed region, run one 1 GiB xfc_copy (the known-size kernel the traffic "
+                         "counters are scaled by when this command runs under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (label sharding across GPUs is design-only); use --gpus 1",
@@ -142,6 +145,15 @@ def main() -> int:
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": DW_UPDATE_TRAFFIC_BYTES.get(args.config)},
     }
+    if args.calibrate:
+        from renee_amd._lib import check, lib
+
+        src = torch.zeros(1 << 29, dtype=torch.float16, device=dev)  # 1 GiB
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        check(lib().xfc_copy(src.data_ptr(), dst.data_ptr(), src.numel() * 2,
+                             torch.cuda.current_stream().cuda_stream), "xfc_copy")
+        torch.cuda.synchronize()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.config, d, args.seed)
     print(json.dumps(out))

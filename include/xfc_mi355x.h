@@ -162,6 +162,14 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw,
              float* values, int64_t* indices,
              void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Plain device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte aligned
+ * pointers).  No counterpart in the reference: it is the kernel of known size against
+ * which the HBM traffic counters (FETCH_SIZE / WRITE_SIZE) of the other kernels are
+ * scaled when profiling, and a convenient way to snapshot W or M on a stream.
+ */
+int xfc_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

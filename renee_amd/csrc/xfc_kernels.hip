@@ -8,6 +8,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 #include "../../include/xfc_mi355x.h"
 #include "pipe_core.hpp"
 
@@ -154,9 +156,11 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
     for (int fm = 0; fm < C::FM; ++fm)
 #pragma unroll
       for (int fn = 0; fn < C::FN; ++fn) words[fm][fn] = 0u;
+    bool has_pos = false;
     if constexpr (MODE == FWD_GRAD) {
       const int s = a.bucket_ptr[nt], e = a.bucket_ptr[nt + 1];
-      if (e > s) {
+      has_pos = e > s;
+      if (has_pos) {
         __syncthreads();  // every wave is done staging the previous tile
         for (int i = threadIdx.x; i < C::BN * (C::BM / 32); i += C::NT) bm[i] = 0u;
         __syncthreads();
@@ -176,44 +180,58 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
     const int h = lane >> 5;
     const int srow = lane >> 3, sch = lane & 7;          // staging read: 8 rows x 8 chunks of 8 labels
     const int col = n0 + wn * C::TN + sch * 8;
+    // The per-element work below is the vector ALU cost of the whole tile (the SIMD cannot overlap it
+    // with MFMAs), so the rare cases -- a tile holding positives, a tile crossing the label count -- are
+    // compiled as separate paths and the common one carries neither.
+    auto body = [&](auto pos_tag, auto edge_tag) {
+      constexpr bool POS = decltype(pos_tag)::value, EDGE = decltype(edge_tag)::value;
 #pragma unroll
-    for (int fm = 0; fm < C::FM; ++fm) {
+      for (int fm = 0; fm < C::FM; ++fm) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < 4; ++q) {
 #pragma unroll
-        for (int fn = 0; fn < C::FN; ++fn) {
-          const int ecol = n0 + wn * C::TN + fn * 32 + (lane & 31);
+          for (int fn = 0; fn < C::FN; ++fn) {
+            const int ecol = n0 + wn * C::TN + fn * 32 + (lane & 31);
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            const int r = 4 * q + rr;
-            float v = a.alpha * acc[fm][fn][r];
-            if constexpr (BETA) {
-              const int erow = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
-              if (erow < a.M && ecol < a.N) v += a.beta * (float)a.out[(int64_t)erow * a.ldo + ecol];
+            for (int rr = 0; rr < 4; ++rr) {
+              const int r = 4 * q + rr;
+              float v = acc[fm][fn][r];
+              if constexpr (BETA) {
+                v *= a.alpha;
+                const int erow = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
+                if (erow < a.M && ecol < a.N) v += a.beta * (float)a.out[(int64_t)erow * a.ldo + ecol];
+              } else if constexpr (MODE == FWD_SIGMOID) {
+                v *= a.alpha;
+              }
+              if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
+              if constexpr (POS) v -= (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
+              if constexpr (EDGE) { if (ecol >= a.N) v = 0.f; }
+              stg[(4 * h + rr) * 64 + fn * 32 + (lane & 31)] = (half_t)v;
             }
-            if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
-            if constexpr (MODE == FWD_GRAD) v -= (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
-            if (ecol >= a.N) v = 0.f;
-            stg[(4 * h + rr) * 64 + fn * 32 + (lane & 31)] = (half_t)v;
           }
-        }
-        // the wave's LDS traffic is ordered: its own writes above are visible to the read below
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        const half8 v8 = *reinterpret_cast<const half8*>(stg + srow * 64 + sch * 8);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
-        if (row < a.M) {
-          half_t* dst = a.out + (int64_t)row * a.ldo + col;
-          if (col + 8 <= a.n_store) {
-            *reinterpret_cast<half8*>(dst) = v8;
-          } else {
+          // the wave's LDS traffic is ordered: its own writes above are visible to the read below
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          const half8 v8 = *reinterpret_cast<const half8*>(stg + srow * 64 + sch * 8);
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
+          if (row < a.M) {
+            half_t* dst = a.out + (int64_t)row * a.ldo + col;
+            if (!EDGE || col + 8 <= a.n_store) {
+              *reinterpret_cast<half8*>(dst) = v8;
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (col + e < a.n_store) dst[e] = v8[e];
+              for (int e = 0; e < 8; ++e)
+                if (col + e < a.n_store) dst[e] = v8[e];
+            }
           }
         }
       }
-    }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    const bool edge = n0 + C::BN > a.N;
+    if (edge) { if (has_pos) body(T{}, T{}); else body(F{}, T{}); }
+    else { if (has_pos) body(T{}, F{}); else body(F{}, F{}); }
   };
   C::run(0, n_items, lds, get, epilogue);
 }
@@ -544,58 +562,72 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
     const int m0 = mt * C::BM, n0 = nt * C::BN;
     const int h = lane >> 5;
     const int srow = lane >> 3, sch = lane & 7;  // staging read: 8 rows x 8 chunks of 8 dims
+    // The tile is walked in NS strips of 8 label rows x 64 dims per wave.  In DW_UPDATE mode the strip's
+    // W and M pieces are fetched DEPTH strips ahead: one strip in flight per wave leaves HBM latency-bound.
+    constexpr int NS = C::FM * 4 * (C::FN / 2);
+    constexpr int DEPTH = 4;
+    auto strip_row = [&](int s) { return m0 + wm * C::TM + (s / (4 * (C::FN / 2))) * 32 + 8 * ((s / (C::FN / 2)) % 4) + srow; };
+    auto strip_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 8; };
+    half8 wq[DEPTH], mq[DEPTH];
+    auto fetch = [&](int s, half8& wv, half8& mv) {
+      const int row = strip_row(s), col = strip_col(s);
+      if (row < a.M && col < a.N) {
+        wv = *reinterpret_cast<const half8*>(a.Wt + (int64_t)row * a.ldw + col);
+        mv = *reinterpret_cast<const half8*>(a.Mo + (int64_t)row * a.ldm + col);
+      }
+    };
+    if constexpr (MODE == DW_UPDATE) {
 #pragma unroll
-    for (int fm = 0; fm < C::FM; ++fm) {
+      for (int s = 0; s < DEPTH && s < NS; ++s) fetch(s, wq[s], mq[s]);
+    }
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+    for (int s = 0; s < NS; ++s) {
+      const int fm = s / (4 * (C::FN / 2)), q = (s / (C::FN / 2)) % 4, fp = s % (C::FN / 2);
 #pragma unroll
-        for (int fp = 0; fp < C::FN / 2; ++fp) {
+      for (int f = 0; f < 2; ++f)
 #pragma unroll
-          for (int f = 0; f < 2; ++f)
+        for (int rr = 0; rr < 4; ++rr)
+          stage[(4 * h + rr) * 64 + f * 32 + (lane & 31)] = acc[fm][2 * fp + f][4 * q + rr];
+      // the wave's own LDS traffic is ordered: the writes above are visible to the reads below
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      const float4v v0 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8);
+      const float4v v1 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8 + 4);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int row = strip_row(s), col = strip_col(s);
+      const bool in = row < a.M && col < a.N;
+      const float g[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      if constexpr (MODE == DW_OUT) {
+        if (in) {
+          float* o = a.out + (int64_t)row * a.ldo + col;
+          float4v o0, o1;
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr)
-              stage[(4 * h + rr) * 64 + f * 32 + (lane & 31)] = acc[fm][2 * fp + f][4 * q + rr];
-          // the wave's own LDS traffic is ordered: the writes above are visible to the reads below
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          const float4v v0 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8);
-          const float4v v1 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8 + 4);
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
-          const int col = n0 + wn * C::TN + fp * 64 + sch * 8;
-          if (row >= a.M || col >= a.N) continue;
-          const float g[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-          if constexpr (MODE == DW_OUT) {
-            float* o = a.out + (int64_t)row * a.ldo + col;
-            float4v o0, o1;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
-            if (a.beta != 0.f) {
-              o0 += a.beta * *reinterpret_cast<const float4v*>(o);
-              o1 += a.beta * *reinterpret_cast<const float4v*>(o + 4);
-            }
-            *reinterpret_cast<float4v*>(o) = o0;
-            *reinterpret_cast<float4v*>(o + 4) = o1;
-          } else {
-            half_t* wp = a.Wt + (int64_t)row * a.ldw + col;
-            half_t* mp = a.Mo + (int64_t)row * a.ldm + col;
-            half8 wv = *reinterpret_cast<const half8*>(wp);
-            half8 mv = *reinterpret_cast<const half8*>(mp);
-            if (a.dw_dump) {
-              float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
-              *reinterpret_cast<float4v*>(d) = v0;
-              *reinterpret_cast<float4v*>(d + 4) = v1;
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const float wf = (float)wv[e];
-              const float gg = g[e] + a.wd * wf;
-              const float mf = a.mu * (float)mv[e] + gg;
-              mv[e] = (half_t)mf;
-              wv[e] = (half_t)(wf - a.lr * mf);
-            }
-            *reinterpret_cast<half8*>(mp) = mv;
-            *reinterpret_cast<half8*>(wp) = wv;
+          for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
+          if (a.beta != 0.f) {
+            o0 += a.beta * *reinterpret_cast<const float4v*>(o);
+            o1 += a.beta * *reinterpret_cast<const float4v*>(o + 4);
           }
+          *reinterpret_cast<float4v*>(o) = o0;
+          *reinterpret_cast<float4v*>(o + 4) = o1;
+        }
+      } else {
+        half8 wv = wq[s % DEPTH], mv = mq[s % DEPTH];
+        if (s + DEPTH < NS) fetch(s + DEPTH, wq[s % DEPTH], mq[s % DEPTH]);
+        if (in) {
+          if (a.dw_dump) {
+            float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
+            *reinterpret_cast<float4v*>(d) = v0;
+            *reinterpret_cast<float4v*>(d + 4) = v1;
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float wf = (float)wv[e];
+            const float gg = g[e] + a.wd * wf;
+            const float mf = a.mu * (float)mv[e] + gg;
+            mv[e] = (half_t)mf;
+            wv[e] = (half_t)(wf - a.lr * mf);
+          }
+          *reinterpret_cast<half8*>(a.Mo + (int64_t)row * a.ldm + col) = mv;
+          *reinterpret_cast<half8*>(a.Wt + (int64_t)row * a.ldw + col) = wv;
         }
       }
     }
@@ -628,6 +660,12 @@ __global__ void __launch_bounds__(256) generic_gemm_kernel(const half_t* __restr
     if (sigmoid) s = sigmoidf_fast(s);
     *p = s;
   }
+}
+
+// Plain copy, 16 bytes per thread step: the known-size kernel that HBM traffic counters are scaled by.
+__global__ void __launch_bounds__(256) copy_kernel(const uint4v* __restrict__ src, uint4v* __restrict__ dst, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
 // SGD-momentum on an fp32 gradient (used when dW was accumulated over micro-batches).
@@ -1058,6 +1096,19 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   if (rc) return rc;
   hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)B), dim3(64), 0, st, a.cand_v, a.cand_i, (int)B, a.n_groups, K,
                      numy, values, indices);
+  return check_launch();
+}
+
+int xfc_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+  if (bytes < 0) return XFC_ERR_INVALID;
+  if (bytes == 0) return XFC_OK;
+  if (!src || !dst) return XFC_ERR_INVALID;
+  if (bytes % 16 || !aligned16(src) || !aligned16(dst)) return XFC_ERR_ALIGN;
+  const int64_t n16 = bytes / 16;
+  int64_t grid = ceil_div(n16, 256);
+  if (grid > 16384) grid = 16384;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<const uint4v*>(src), reinterpret_cast<uint4v*>(dst), n16);
   return check_launch();
 }
 

@@ -1,0 +1,102 @@
+"""Full BASELINE sizes.  The CPU oracle cannot finish these in seconds, so the
+checks are (i) the same fp32 formulation evaluated with torch on the GPU in
+label chunks for quantities that reduce over all labels (dX, top-5), (ii) the
+CPU oracle on sampled label rows / columns for G, dW and the update, and
+(iii) size-independent properties (linearity of dX in the loss scale, sign
+structure of G, zeroed pad columns)."""
+import pytest
+import torch
+
+from oracle import xfc_oracle as O
+from renee_amd import XFCLayer, synth
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def rel(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float((a - b).norm() / b.norm())
+
+
+def _fullsize_step(dev, cfg, sample=384):
+    c = synth.CONFIGS[cfg]
+    B, L, d = c["B"], c["L"], synth.D_MODEL
+    print(f"cfg{cfg}: B={B} L={L}", flush=True)
+    lay = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=1e-4, seed=cfg)
+    X = synth.make_X(B, d, cfg, dev).half()
+    P = synth.make_positives(B, L, c["kmax"], c["kmean"], c["zipf"], cfg)
+    rp, ci = torch.from_numpy(P.rowptr).to(dev), torch.from_numpy(P.colidx).to(dev)
+    g = torch.Generator().manual_seed(cfg)
+    # sampled labels: the Zipf head, the ragged tail, every positive label of a few rows, and random ones
+    pick = torch.cat([torch.arange(0, 64), torch.arange(L - 64, L), torch.from_numpy(P.colidx[:64]).long(),
+                      torch.randint(0, L, (sample,), generator=g)]).unique()
+    W0 = lay.xfc_weight[pick.to(dev)].float().cpu()
+    G = lay.fwd_grad(X, rowptr=rp, colidx=ci)
+    px, py = P.coo()
+    # G on the sampled label columns vs the CPU oracle
+    Zs = O.logits(X.float().cpu(), W0)
+    Ys = torch.zeros(B, len(pick))
+    lut = {int(l): j for j, l in enumerate(pick.tolist())}
+    for r, l in zip(px.tolist(), py.tolist()):
+        if l in lut:
+            Ys[r, lut[l]] = 1.0
+    Gs_ref = torch.sigmoid(Zs) - Ys
+    Gs = G[:, pick.to(dev)].float().cpu()
+    assert rel(Gs, Gs_ref) <= TOL
+    assert ((Gs < 0) == (Ys > 0)).all()
+    if lay.ldg > L:
+        assert float(lay.outsoft[:B, L:].abs().max()) == 0.0
+    # dX: same formulation with torch fp32 on the GPU, in label chunks, from the kernel's own G
+    dX = lay.dx(B, scale=2.0).clone()
+    ref = torch.zeros(B, d, device=dev)
+    step = 1 << 17
+    for l0 in range(0, L, step):
+        l1 = min(L, l0 + step)
+        ref += G[:, l0:l1].float() @ lay.xfc_weight[l0:l1].float()
+    assert rel(dX, 2.0 * ref) <= TOL
+    assert torch.allclose(lay.dx(B, scale=1.0) * 2.0, dX, rtol=1e-6, atol=0)
+    # dW + update on the sampled labels vs the CPU oracle (from the kernel's G, so only this kernel is judged)
+    M0 = lay.momentum_buffer[pick.to(dev)].float().cpu()
+    Gs16 = G[:, pick.to(dev)].float().cpu()
+    lay.dw_update(X)
+    dW_ref = O.dw(Gs16, X.float().cpu())
+    W_ref, M_ref = O.sgd_momentum(W0, M0, dW_ref, 0.05, 0.9, 1e-4)
+    assert rel(lay.momentum_buffer[pick.to(dev)], M_ref) <= TOL
+    assert rel(lay.xfc_weight[pick.to(dev)], W_ref) <= TOL
+    return lay, X
+
+
+def test_config2_headline_shape(dev):
+    _fullsize_step(dev, 2)
+
+
+def test_config3_ragged_labels_and_top5(dev):
+    lay, X = _fullsize_step(dev, 3)
+    B, L = X.shape[0], lay.numy
+    v, i = lay.topk(X, 5)
+    # reference: fp32 logits on the GPU in label chunks, running top-5 with a stable sort (lowest id first)
+    best_v = torch.full((B, 5), float("-inf"), device=dev)
+    best_i = torch.zeros(B, 5, dtype=torch.int64, device=dev)
+    step = 1 << 17
+    for l0 in range(0, L, step):
+        l1 = min(L, l0 + step)
+        Z = X.float() @ lay.xfc_weight[l0:l1].float().t()
+        cv = torch.cat([best_v, Z], 1)
+        cidx = torch.cat([best_i, torch.arange(l0, l1, device=dev).expand(B, -1)], 1)
+        sv, sp = torch.sort(cv, dim=1, descending=True, stable=True)
+        best_v, best_i = sv[:, :5], torch.gather(cidx, 1, sp[:, :5])
+    scale = float(best_v.abs().max())
+    assert torch.allclose(v, best_v, rtol=0, atol=2e-5 * scale)
+    mism = (i != best_i)
+    # the two fp32 evaluations differ in summation order: allow swaps only between near-equal scores
+    if mism.any():
+        for b, j in mism.nonzero().tolist():
+            other = best_v[b, min(j + 1, 4)] if j < 4 else best_v[b, j - 1]
+            gap = min(abs(float(best_v[b, j] - other)), abs(float(best_v[b, max(j - 1, 0)] - best_v[b, j])) or 1e9)
+            assert gap <= 1e-5 * scale, (b, j)
+    assert float(mism.float().mean()) < 0.01
+
+
+def test_config4_streaming_shape(dev):
+    _fullsize_step(dev, 4, sample=128)
