@@ -108,8 +108,12 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
 enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2 };
 
 using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true>;
-constexpr int FWD_AUX_BYTES = FwdCore::BN * (FwdCore::BM / 32) * 4;  // bitmap, then 8 x 64 halves of staging per wave
-static_assert(FWD_AUX_BYTES >= FwdCore::NW * 512 * 2 && FwdCore::FN == 2, "staging fits the bitmap area");
+// beside the ring: the tile's positives bitmap, later reused as store staging (8 rows x TN labels per wave)
+constexpr int FWD_STG_HALVES = 8 * FwdCore::TN;
+constexpr int FWD_BITMAP_BYTES = FwdCore::BN * (FwdCore::BM / 32) * 4;
+constexpr int FWD_AUX_BYTES = FWD_BITMAP_BYTES > FwdCore::NW * FWD_STG_HALVES * 2 ? FWD_BITMAP_BYTES
+                                                                                    : FwdCore::NW * FWD_STG_HALVES * 2;
+static_assert(FwdCore::FN % 2 == 0, "staging read-back walks 64-label pieces");
 constexpr int FWD_LDS_BYTES = FwdCore::LDS_BYTES + FWD_AUX_BYTES;
 
 struct FwdArgs {
@@ -129,13 +133,13 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
   using C = FwdCore;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
-  // 4 KB beside the ring: first the tile's positives bitmap, then per-wave store staging
+  // beside the ring: first the tile's positives bitmap, then per-wave store staging
   uint32_t* bm = reinterpret_cast<uint32_t*>(smem_raw + C::LDS_BYTES);
   const int G = gridDim.x, w = blockIdx.x;
   const int n_items = (a.n_ids - w + G - 1) / G;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
-  half_t* stg = reinterpret_cast<half_t*>(bm) + wave * 512;  // 8 rows x 64 labels
+  half_t* stg = reinterpret_cast<half_t*>(bm) + wave * FWD_STG_HALVES;  // 8 rows x TN labels
 
   auto get = [&](int item, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
     int mt, nt;
@@ -178,8 +182,7 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
       }
     }
     const int h = lane >> 5;
-    const int srow = lane >> 3, sch = lane & 7;          // staging read: 8 rows x 8 chunks of 8 labels
-    const int col = n0 + wn * C::TN + sch * 8;
+    constexpr int CHS = C::TN / 8;  // 16-byte chunks per staged row
     // The per-element work below is the vector ALU cost of the whole tile (the SIMD cannot overlap it
     // with MFMAs), so the rare cases -- a tile holding positives, a tile crossing the label count -- are
     // compiled as separate paths and the common one carries neither.
@@ -206,24 +209,30 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
               if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
               if constexpr (POS) v -= (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
               if constexpr (EDGE) { if (ecol >= a.N) v = 0.f; }
-              stg[(4 * h + rr) * 64 + fn * 32 + (lane & 31)] = (half_t)v;
+              stg[(4 * h + rr) * C::TN + fn * 32 + (lane & 31)] = (half_t)v;
             }
           }
-          // the wave's LDS traffic is ordered: its own writes above are visible to the read below
+          // the wave's LDS traffic is ordered: its own writes above are visible to the reads below
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          const half8 v8 = *reinterpret_cast<const half8*>(stg + srow * 64 + sch * 8);
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
-          if (row < a.M) {
-            half_t* dst = a.out + (int64_t)row * a.ldo + col;
-            if (!EDGE || col + 8 <= a.n_store) {
-              *reinterpret_cast<half8*>(dst) = v8;
-            } else {
 #pragma unroll
-              for (int e = 0; e < 8; ++e)
-                if (col + e < a.n_store) dst[e] = v8[e];
+          for (int p = 0; p < C::FN / 2; ++p) {
+            const int cid = lane + 64 * p;
+            const int srow = cid / CHS, sch = cid % CHS;
+            const half8 v8 = *reinterpret_cast<const half8*>(stg + srow * C::TN + sch * 8);
+            const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
+            const int col = n0 + wn * C::TN + sch * 8;
+            if (row < a.M) {
+              half_t* dst = a.out + (int64_t)row * a.ldo + col;
+              if (!EDGE || col + 8 <= a.n_store) {
+                *reinterpret_cast<half8*>(dst) = v8;
+              } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  if (col + e < a.n_store) dst[e] = v8[e];
+              }
             }
           }
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
       }
     };
