@@ -36,28 +36,38 @@ __device__ __forceinline__ void xcd_map(int id, int n_inner, int& inner, int& ou
 // ---------------------------------------------------------------------------------------------
 // One workgroup.  Input is CSR (rowptr/colidx, pos_x == nullptr) or COO (pos_x/pos_y int64).
 // Output: bucket_ptr[n_tiles+1] and (ent_row, ent_col)[nnz] grouped by col / tile_w.
-// Pairs whose row or column is out of range are dropped.  cursor[n_tiles] is scratch.
+// Pairs whose row or column is out of range are dropped.  The per-tile counters live in LDS when
+// they fit (IN_LDS, n_tiles <= BUCKET_LDS_TILES) and in the global scratch array `cursor` otherwise.
+constexpr int BUCKET_LDS_TILES = 12288;
+
+template <bool IN_LDS>
 __global__ void __launch_bounds__(1024) bucket_positives_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ colidx, const int64_t* __restrict__ pos_x,
     const int64_t* __restrict__ pos_y, int64_t nnz, int B, int64_t L, int tile_w, int n_tiles,
-    int32_t* __restrict__ bucket_ptr, int32_t* __restrict__ cursor, int32_t* __restrict__ ent_row,
+    int32_t* __restrict__ bucket_ptr, int32_t* __restrict__ cursor_g, int32_t* __restrict__ ent_row,
     int32_t* __restrict__ ent_col) {
   __shared__ int32_t part[1024];
+  extern __shared__ int32_t cursor_l[];
+  int32_t* cursor = IN_LDS ? cursor_l : cursor_g;
   const int t = threadIdx.x;
   for (int i = t; i < n_tiles; i += 1024) cursor[i] = 0;
   __syncthreads();
-  if (pos_x) {
-    for (int64_t p = t; p < nnz; p += 1024) {
-      const int64_t r = pos_x[p], c = pos_y[p];
-      if (r >= 0 && r < B && c >= 0 && c < L) atomicAdd(&cursor[(int)(c / tile_w)], 1);
-    }
-  } else {
-    for (int b = t; b < B; b += 1024)
-      for (int p = rowptr[b]; p < rowptr[b + 1]; ++p) {
-        const int64_t c = colidx[p];
-        if (c >= 0 && c < L) atomicAdd(&cursor[(int)(c / tile_w)], 1);
+  // pass 0 counts, pass 1 places
+  auto walk = [&](auto visit) {
+    if (pos_x) {
+      for (int64_t p = t; p < nnz; p += 1024) {
+        const int64_t r = pos_x[p], c = pos_y[p];
+        if (r >= 0 && r < B && c >= 0 && c < L) visit((int)r, (int)c);
       }
-  }
+    } else {
+      for (int b = t; b < B; b += 1024)
+        for (int p = rowptr[b]; p < rowptr[b + 1]; ++p) {
+          const int64_t c = colidx[p];
+          if (c >= 0 && c < L) visit(b, (int)c);
+        }
+    }
+  };
+  walk([&](int, int c) { atomicAdd(&cursor[c / tile_w], 1); });
   __syncthreads();
   const int per = (n_tiles + 1023) / 1024;
   const int lo = t * per, hi = min(n_tiles, lo + per);
@@ -66,7 +76,7 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
   part[t] = s;
   __syncthreads();
   for (int off = 1; off < 1024; off <<= 1) {
-    int v = t >= off ? part[t - off] : 0;
+    const int v = t >= off ? part[t - off] : 0;
     __syncthreads();
     part[t] += v;
     __syncthreads();
@@ -80,26 +90,11 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
   }
   if (t == 1023) bucket_ptr[n_tiles] = part[1023];
   __syncthreads();
-  if (pos_x) {
-    for (int64_t p = t; p < nnz; p += 1024) {
-      const int64_t r = pos_x[p], c = pos_y[p];
-      if (r >= 0 && r < B && c >= 0 && c < L) {
-        const int at = atomicAdd(&cursor[(int)(c / tile_w)], 1);
-        ent_row[at] = (int)r;
-        ent_col[at] = (int)c;
-      }
-    }
-  } else {
-    for (int b = t; b < B; b += 1024)
-      for (int p = rowptr[b]; p < rowptr[b + 1]; ++p) {
-        const int64_t c = colidx[p];
-        if (c >= 0 && c < L) {
-          const int at = atomicAdd(&cursor[(int)(c / tile_w)], 1);
-          ent_row[at] = b;
-          ent_col[at] = (int)c;
-        }
-      }
-  }
+  walk([&](int r, int c) {
+    const int at = atomicAdd(&cursor[c / tile_w], 1);
+    ent_row[at] = r;
+    ent_col[at] = c;
+  });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -956,9 +951,14 @@ static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw,
   BucketWs bk = carve_bucket_ws(ws, L, nnz);
   const int n_tiles = (int)round_up(ceil_div(L, FwdCore::BN), 8);
   const bool coo = pos_x != nullptr;
-  hipLaunchKernelGGL(bucket_positives_kernel, dim3(1), dim3(1024), 0, st, coo ? nullptr : rowptr,
-                     coo ? nullptr : colidx, coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L,
-                     FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
+  if (n_tiles <= BUCKET_LDS_TILES)
+    hipLaunchKernelGGL(bucket_positives_kernel<true>, dim3(1), dim3(1024), n_tiles * 4, st, coo ? nullptr : rowptr,
+                       coo ? nullptr : colidx, coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L,
+                       FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
+  else
+    hipLaunchKernelGGL(bucket_positives_kernel<false>, dim3(1), dim3(1024), 0, st, coo ? nullptr : rowptr,
+                       coo ? nullptr : colidx, coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L,
+                       FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
   int rc = check_launch();
   if (rc) return rc;
   // label columns L .. round_up(L, 8) are written as zero so that G can be read in 16-byte
