@@ -76,7 +76,7 @@ __device__ __forceinline__ int kc_swz(int row) {
 // transposing read touches then sit in four different 64-byte bank groups.
 __device__ __forceinline__ int mc_swz(int k) { return (k & 3) << 2; }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_, bool ACC_AGPR_ = false>
 struct PipeCore {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
@@ -215,21 +215,44 @@ struct PipeCore {
       else f.b[fn] = frag_mc<BN>(sb, wn * TN + fn * 32, kk, lane);
     }
   }
+  // ACC_AGPR pins the accumulators to the accumulation register file ("a" constraint; the compiler only
+  // picks that form by itself above 256 registers).  With the accumulators in ordinary vector registers
+  // a SIMD's MFMAs and its global->LDS fetches serialise more (microbenchmark: one stage of fetches plus
+  // 32 MFMAs per wave, 1.19 ms-equivalents against 0.83 with AGPR accumulators; 0.69 / 0.61 for either
+  // alone), but the AGPR form leaves only 128 ordinary registers and costs a copy per accumulator read,
+  // so it pays only where the epilogue is trivial (dX).  Being inline asm, the instruction is invisible
+  // to the compiler's MFMA hazard bookkeeping: settle() supplies the wait states an MFMA result needs
+  // before ordinary code may read it, zero() those between an accumulator write and its use as source C.
   __device__ __forceinline__ static void mfma_all(const Frags& f, float16v (&acc)[FM][FN]) {
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
-      for (int fn = 0; fn < FN; ++fn)
-        acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[fm], f.b[fn], acc[fm][fn], 0, 0, 0);
+      for (int fn = 0; fn < FN; ++fn) {
+        if constexpr (ACC_AGPR_)
+          asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[fm][fn]) : "v"(f.a[fm]), "v"(f.b[fn]));
+        else
+          acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[fm], f.b[fn], acc[fm][fn], 0, 0, 0);
+      }
   }
-
+  // At least 18 idle issue slots must separate an MFMA from a non-MFMA read or write of its destination.
+  __device__ __forceinline__ static void settle(float16v (&acc)[FM][FN]) {
+    if constexpr (ACC_AGPR_) {
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+        for (int fn = 0; fn < FN; ++fn)
+          asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[fm][fn]));
+    }
+  }
   __device__ __forceinline__ static void zero(float16v (&acc)[FM][FN]) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j)
+      for (int j = 0; j < FN; ++j) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        if constexpr (ACC_AGPR_) asm volatile("s_nop 3" : "+a"(acc[i][j]));  // accumulator write -> MFMA source C
+      }
   }
 
   // Walks the work items [item_begin, item_end) of this workgroup.
@@ -334,6 +357,7 @@ struct PipeCore {
         cur = nxt;
         c_slot = n_slot;
       }
+      settle(acc);
       epilogue(item, acc);
       zero(acc);
       drain_all = true;

@@ -289,8 +289,8 @@ __device__ __forceinline__ void topk_insert(float* lv, int32_t* li, int K, float
   li[p] = i;
 }
 
-// Out of line on purpose: inlined 128 times into the filter, the compiler merges the bodies and the
-// register pressure of the whole epilogue explodes.
+// Out of line on purpose: inlined 128 times into the filter, the bodies get merged by the compiler and
+// the register pressure of the whole epilogue explodes (about 180 spilled registers against 2).
 __device__ __attribute__((noinline)) void topk_push(TopkLds& S, int row, float v, int col) {
   const int slot = atomicAdd(&S.cnt[row], 1);
   if (slot < TOPK_CAP) { S.buf_v[row][slot] = v; S.buf_i[row][slot] = col; }
@@ -439,7 +439,7 @@ __global__ void __launch_bounds__(64) topk_merge_kernel(const float* __restrict_
 // ---------------------------------------------------------------------------------------------
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
-using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false>;
+using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, true>;  // accumulators in AGPRs
 constexpr int DX_LDS_BYTES = DxCore::LDS_BYTES;
 
 struct DxArgs {
