@@ -82,17 +82,22 @@ int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out
  * dl_base.py:934-936), in any order.
  * G has leading dimension ldg >= L, a multiple of 8; the columns
  * L .. round_up(L,8)-1 are written as zero (xfc_dx / xfc_dw_update rely on it).
+ * If `loss` is non-NULL it receives the summed BCE-with-logits loss of the batch,
+ *   sum softplus(z) - sum z[positives]          (fp32; Algorithm 1 of the paper,
+ * dl_base.py:578-583, which the reference evaluates on one step in 100), from the same
+ * pass; positives count once each (the reference's indexed sum would count a duplicated
+ * pair twice).  NULL is the --noloss path and costs nothing.
  * Workspace: xfc_fwd_grad_workspace_bytes(L, nnz) bytes.
  */
 size_t xfc_fwd_grad_workspace_bytes(int64_t L, int64_t nnz);
 int xfc_fwd_grad_csr(const void* X, int64_t ldx, const void* W, int64_t ldw,
                      const int32_t* rowptr, const int32_t* colidx,
                      void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, int64_t nnz,
-                     void* workspace, size_t workspace_bytes, void* stream);
+                     float* loss, void* workspace, size_t workspace_bytes, void* stream);
 int xfc_fwd_grad_coo(const void* X, int64_t ldx, const void* W, int64_t ldw,
                      const int64_t* pos_x, const int64_t* pos_y, int64_t nnz,
                      void* G, int64_t ldg, int64_t B, int64_t L, int64_t d,
-                     void* workspace, size_t workspace_bytes, void* stream);
+                     float* loss, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * dX[B x d] (fp32) = scale * G[B x L] . W[L x d].

@@ -118,12 +118,13 @@ struct FwdArgs {
   int M, N, K, n_store;             // columns N <= c < n_store are written as zero
   float alpha, beta;
   const int32_t* bucket_ptr; const int32_t* ent_row; const int32_t* ent_col;
+  float* loss_part;                 // FWD_GRAD with LOSS: one partial sum per workgroup
   int tiles_m, tiles_n, n_ids;      // n_ids = tiles_m * round_up(tiles_n, 8)
 };
 
 // Persistent: workgroup w takes tile ids w, w + gridDim.x, ... (gridDim.x a multiple of 8, so an
 // id keeps its XCD and the row tiles of one label tile run side by side on one L2).
-template <int MODE, bool BETA>
+template <int MODE, bool BETA, bool LOSS = false>
 __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
   using C = FwdCore;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
@@ -135,6 +136,7 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WN, wn = wave % C::WN;
   half_t* stg = reinterpret_cast<half_t*>(bm) + wave * FWD_STG_HALVES;  // 8 rows x TN labels
+  float loss_acc = 0.f;  // LOSS: this lane's share of sum softplus(z) - sum z[positives]
 
   auto get = [&](int item, typename C::Operand& oa, typename C::Operand& ob, int& kb, int& ke) {
     int mt, nt;
@@ -183,6 +185,7 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
     // compiled as separate paths and the common one carries neither.
     auto body = [&](auto pos_tag, auto edge_tag) {
       constexpr bool POS = decltype(pos_tag)::value, EDGE = decltype(edge_tag)::value;
+      float tile_loss = 0.f;
 #pragma unroll
       for (int fm = 0; fm < C::FM; ++fm) {
 #pragma unroll
@@ -201,11 +204,22 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
               } else if constexpr (MODE == FWD_SIGMOID) {
                 v *= a.alpha;
               }
+              if constexpr (LOSS) {
+                // softplus(z) = max(z,0) + log(1 + e^-|z|), minus z where the label is positive (dl_base.py:578-583)
+                const int erow = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
+                float t = fmaxf(v, 0.f) + 0.69314718f * __log2f(1.0f + __expf(-fabsf(v)));
+                if constexpr (POS) t -= v * (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
+                if constexpr (EDGE) t = (erow < a.M && ecol < a.N) ? t : 0.f;
+                tile_loss += t;
+              }
               if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
               if constexpr (POS) v -= (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
               if constexpr (EDGE) { if (ecol >= a.N) v = 0.f; }
               stg[(4 * h + rr) * C::TN + fn * 32 + (lane & 31)] = (half_t)v;
             }
+            // with the loss terms the scheduler otherwise interleaves dozens of elements to hide the
+            // transcendental latency and spills hundreds of registers
+            if constexpr (LOSS) __builtin_amdgcn_sched_barrier(0);
           }
           // the wave's LDS traffic is ordered: its own writes above are visible to the reads below
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -230,14 +244,38 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
       }
+      if constexpr (LOSS) loss_acc += tile_loss;
     };
     using T = std::true_type;
     using F = std::false_type;
-    const bool edge = n0 + C::BN > a.N;
+    const bool edge = n0 + C::BN > a.N || (LOSS && m0 + C::BM > a.M);
     if (edge) { if (has_pos) body(T{}, T{}); else body(F{}, T{}); }
     else { if (has_pos) body(T{}, F{}); else body(F{}, F{}); }
   };
   C::run(0, n_items, lds, get, epilogue);
+  if constexpr (LOSS) {
+    // deterministic: lanes -> wave (butterfly), waves -> workgroup (LDS, fixed order), one partial per workgroup
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) loss_acc += __shfl_xor(loss_acc, off, 64);
+    float* red = reinterpret_cast<float*>(bm);
+    __syncthreads();
+    if (lane == 0) red[wave] = loss_acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float t = 0.f;
+      for (int i = 0; i < C::NW; ++i) t += red[i];
+      a.loss_part[w] = t;
+    }
+  }
+}
+
+// Sum of the per-workgroup loss partials, in double, in index order.
+__global__ void __launch_bounds__(64) loss_reduce_kernel(const float* __restrict__ part, int n, float* __restrict__ out) {
+  double t = 0.0;
+  for (int i = threadIdx.x; i < n; i += 64) t += (double)part[i];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
+  if (threadIdx.x == 0) *out = (float)t;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -738,14 +776,16 @@ int num_cus() {
   return n;
 }
 
+constexpr size_t LOSS_PART_BYTES = 4096;  // one float per forward workgroup (at most 1024)
 struct BucketWs {
   int32_t *bucket_ptr, *cursor, *ent_row, *ent_col;
+  float* loss_part;
 };
 
 size_t bucket_ws_bytes(int64_t L, int64_t nnz) {
   const int64_t n_tiles = round_up(ceil_div(L, FwdCore::BN), 8);
   return (size_t)round_up((n_tiles + 1) * 4, 256) + (size_t)round_up(n_tiles * 4, 256) +
-         2 * (size_t)round_up((nnz > 0 ? nnz : 1) * 4, 256);
+         2 * (size_t)round_up((nnz > 0 ? nnz : 1) * 4, 256) + LOSS_PART_BYTES;
 }
 
 BucketWs carve_bucket_ws(void* ws, int64_t L, int64_t nnz) {
@@ -755,18 +795,21 @@ BucketWs carve_bucket_ws(void* ws, int64_t L, int64_t nnz) {
   b.bucket_ptr = reinterpret_cast<int32_t*>(p); p += round_up((n_tiles + 1) * 4, 256);
   b.cursor = reinterpret_cast<int32_t*>(p); p += round_up(n_tiles * 4, 256);
   b.ent_row = reinterpret_cast<int32_t*>(p); p += round_up((nnz > 0 ? nnz : 1) * 4, 256);
-  b.ent_col = reinterpret_cast<int32_t*>(p);
+  b.ent_col = reinterpret_cast<int32_t*>(p); p += round_up((nnz > 0 ? nnz : 1) * 4, 256);
+  b.loss_part = reinterpret_cast<float*>(p);
   return b;
 }
 
 int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, half_t* out, int64_t ldo, int M,
-               int N, int K, int n_store, float alpha, float beta, const BucketWs* bk, hipStream_t st) {
+               int N, int K, int n_store, float alpha, float beta, const BucketWs* bk, hipStream_t st,
+               float* loss_part = nullptr, float* loss_out = nullptr) {
   FwdArgs a;
   a.X = X; a.ldx = ldx; a.W = W; a.ldw = ldw; a.out = out; a.ldo = ldo;
   a.M = M; a.N = N; a.K = K; a.n_store = n_store; a.alpha = alpha; a.beta = beta;
   a.bucket_ptr = bk ? bk->bucket_ptr : nullptr;
   a.ent_row = bk ? bk->ent_row : nullptr;
   a.ent_col = bk ? bk->ent_col : nullptr;
+  a.loss_part = loss_part;
   a.tiles_m = ceil_div(M, FwdCore::BM);
   a.tiles_n = ceil_div(n_store, FwdCore::BN);
   const int64_t ids = (int64_t)a.tiles_m * round_up(a.tiles_n, 8);
@@ -776,6 +819,13 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   int64_t grid = (int64_t)round_up(num_cus(), 8);  // one resident workgroup per CU
   if (grid > ids) grid = ids;                    // ids is a multiple of 8
   dim3 g((unsigned)grid), b(FwdCore::NT);
+  if (mode == FWD_GRAD && loss_part) {
+    launch_k(fwd_kernel<FWD_GRAD, false, true>, g, b, FWD_LDS_BYTES, st, a);
+    int rc = check_launch();
+    if (rc) return rc;
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(64), 0, st, loss_part, (int)grid, loss_out);
+    return check_launch();
+  }
   if (mode == FWD_GRAD) launch_k(fwd_kernel<FWD_GRAD, false>, g, b, FWD_LDS_BYTES, st, a);
   else if (mode == FWD_SIGMOID && beta != 0.f) launch_k(fwd_kernel<FWD_SIGMOID, true>, g, b, FWD_LDS_BYTES, st, a);
   else if (mode == FWD_SIGMOID) launch_k(fwd_kernel<FWD_SIGMOID, false>, g, b, FWD_LDS_BYTES, st, a);
@@ -939,7 +989,8 @@ size_t xfc_fwd_grad_workspace_bytes(int64_t L, int64_t nnz) {
 
 static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw, const int32_t* rowptr,
                          const int32_t* colidx, const int64_t* pos_x, const int64_t* pos_y, int64_t nnz, void* G,
-                         int64_t ldg, int64_t B, int64_t L, int64_t d, void* ws, size_t ws_bytes, hipStream_t st) {
+                         int64_t ldg, int64_t B, int64_t L, int64_t d, float* loss, void* ws, size_t ws_bytes,
+                         hipStream_t st) {
   if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d) || nnz < 0 || nnz > 0x7fffffff) return XFC_ERR_INVALID;
   if (B == 0 || L == 0) return XFC_OK;
   if (!X || !W || !G || d <= 0) return XFC_ERR_INVALID;
@@ -965,25 +1016,25 @@ static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw,
   // pieces along the label axis by the dX and dW kernels (ldg is a multiple of 8, so they exist)
   const int64_t n_store = round_up(L, 8);
   return launch_fwd(FWD_GRAD, (const half_t*)X, ldx, (const half_t*)W, ldw, (half_t*)G, ldg, (int)B, (int)L, (int)d,
-                    (int)n_store, 1.0f, 0.0f, &bk, st);
+                    (int)n_store, 1.0f, 0.0f, &bk, st, loss ? bk.loss_part : nullptr, loss);
 }
 
 int xfc_fwd_grad_csr(const void* X, int64_t ldx, const void* W, int64_t ldw, const int32_t* rowptr,
                      const int32_t* colidx, void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, int64_t nnz,
-                     void* workspace, size_t workspace_bytes, void* stream) {
+                     float* loss, void* workspace, size_t workspace_bytes, void* stream) {
   if (B > 0 && !rowptr) return XFC_ERR_INVALID;
-  return fwd_grad_impl(X, ldx, W, ldw, rowptr, colidx, nullptr, nullptr, nnz, G, ldg, B, L, d, workspace,
+  return fwd_grad_impl(X, ldx, W, ldw, rowptr, colidx, nullptr, nullptr, nnz, G, ldg, B, L, d, loss, workspace,
                        workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
 int xfc_fwd_grad_coo(const void* X, int64_t ldx, const void* W, int64_t ldw, const int64_t* pos_x, const int64_t* pos_y,
-                     int64_t nnz, void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, void* workspace,
+                     int64_t nnz, void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, float* loss, void* workspace,
                      size_t workspace_bytes, void* stream) {
   if (nnz > 0 && !(pos_x && pos_y)) return XFC_ERR_INVALID;
   // an empty list still goes through the bucket pass (it zeroes the bucket table)
   static const int64_t dummy = 0;
   return fwd_grad_impl(X, ldx, W, ldw, nullptr, nullptr, pos_x ? pos_x : &dummy, pos_y ? pos_y : &dummy, nnz, G, ldg, B,
-                       L, d, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+                       L, d, loss, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
 size_t xfc_dx_workspace_bytes(int64_t B, int64_t L, int64_t d) { return xfc_gemm_workspace_bytes(B, d, L); }
@@ -1058,7 +1109,7 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int
   if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
   const size_t off = (size_t)round_up(xfc_fwd_grad_workspace_bytes(L, nnz), 256);
   unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
-  int rc = xfc_fwd_grad_csr(X, ldx, W, ldw, rowptr, colidx, G, ldg, B, L, d, nnz, ws, off, stream);
+  int rc = xfc_fwd_grad_csr(X, ldx, W, ldw, rowptr, colidx, G, ldg, B, L, d, nnz, nullptr, ws, off, stream);
   if (rc) return rc;
   rc = xfc_dx(G, ldg, W, ldw, dX, lddx, B, L, d, scale, ws + off, workspace_bytes - off, stream);
   if (rc) return rc;

@@ -164,8 +164,15 @@ class XFCLayer:
         check(rc, "xfc_topk")
         return vals, inds
 
-    def fwd_grad(self, embed, pos_x=None, pos_y=None, rowptr=None, colidx=None) -> torch.Tensor:
-        """G = sigmoid(embed . W^T) - Y into outsoft (dl_base.py:591-594); returns the (batch, numy) view."""
+    def fwd_grad(self, embed, pos_x=None, pos_y=None, rowptr=None, colidx=None,
+                 loss_out: torch.Tensor | None = None) -> torch.Tensor:
+        """G = sigmoid(embed . W^T) - Y into outsoft (dl_base.py:591-594); returns the (batch, numy) view.
+        With loss_out (a one-element float32 tensor) the summed BCE loss of the batch
+        (dl_base.py:578-583) is produced by the same pass."""
+        if loss_out is not None:
+            _require(loss_out.dtype == torch.float32 and loss_out.numel() == 1 and loss_out.device == self.device,
+                     "loss_out must be a one-element float32 tensor on the layer's device")
+        lp = None if loss_out is None else loss_out.data_ptr()
         x = self._x16(embed)
         bsz = x.shape[0]
         G = self._g_view(bsz)
@@ -179,7 +186,7 @@ class XFCLayer:
                 _require(rowptr.numel() == bsz + 1, "rowptr must have batch+1 entries")
                 rc = L.xfc_fwd_grad_csr(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                         rowptr.data_ptr(), colidx.data_ptr(), G.data_ptr(), self.ldg,
-                                        bsz, self.numy, self.dims, nnz, ws.data_ptr(), ws.numel(), _stream(x))
+                                        bsz, self.numy, self.dims, nnz, lp, ws.data_ptr(), ws.numel(), _stream(x))
             else:
                 if nnz:
                     _require(pos_x.dtype == torch.int64 and pos_y.dtype == torch.int64, "COO must be int64", TypeError)
@@ -187,7 +194,7 @@ class XFCLayer:
                     pos_x, pos_y = pos_x.contiguous(), pos_y.contiguous()
                 rc = L.xfc_fwd_grad_coo(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                         pos_x.data_ptr() if nnz else None, pos_y.data_ptr() if nnz else None, nnz,
-                                        G.data_ptr(), self.ldg, bsz, self.numy, self.dims,
+                                        G.data_ptr(), self.ldg, bsz, self.numy, self.dims, lp,
                                         ws.data_ptr(), ws.numel(), _stream(x))
         check(rc, "xfc_fwd_grad")
         return G[:, : self.numy]

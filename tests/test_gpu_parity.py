@@ -289,3 +289,23 @@ def test_step_under_graph_capture(dev):
         assert torch.equal(graphed.xfc_weight, eager.xfc_weight)
         assert torch.equal(graphed.momentum_buffer, eager.momentum_buffer)
         assert torch.equal(graphed.grad_input[:B], ge)
+
+
+@pytest.mark.parametrize("B,L,d", [(64, 1000, 64), (300, 70001, 128), (512, 8192, 768)])
+def test_fused_loss(dev, B, L, d):
+    """Summed BCE-with-logits loss from the forward pass (dl_base.py:578-583) against the oracle and
+    against BCEWithLogitsLoss(reduction='sum'); G must be unchanged by asking for the loss."""
+    X, W, P = _problem(B, L, d, seed=3)
+    px, py = P.coo()
+    lay = XFCLayer(L, d, B, dev, weight=W)
+    loss = torch.zeros(1, device=dev)
+    G1 = lay.fwd_grad(X.to(dev), px.to(dev), py.to(dev), loss_out=loss).clone()
+    G0 = lay.fwd_grad(X.to(dev), px.to(dev), py.to(dev))
+    assert torch.equal(G0, G1)
+    Z = O.logits(X.float(), W.float())
+    want = float(O.sampled_loss(Z.double(), px, py))
+    Y = torch.zeros(B, L, dtype=torch.float64)
+    Y[px, py] = 1.0
+    bce = float(torch.nn.BCEWithLogitsLoss(reduction="sum")(Z.double(), Y))
+    assert abs(want - bce) <= 1e-6 * abs(bce)  # the oracle follows the reference and sums in float32
+    assert abs(float(loss) - bce) <= 1e-5 * abs(bce)
