@@ -39,6 +39,14 @@ const char* xfc_strerror(int code);
 int xfc_abi_version(void);
 
 /*
+ * Optional set-up for the calling thread's current device: raises the dynamic-LDS limit of
+ * every kernel and reads the device's CU count, which the entry points otherwise do on
+ * their first launch.  Call it once per device before capturing launches into a graph.
+ * No counterpart in the reference (its kernels fit the default shared-memory limit).
+ */
+int xfc_init(void);
+
+/*
  * The six-argument fused GEMM of the reference extension:
  *   xfc_gemm(mat_in1, mat_in2, mat_out, alpha, beta, apply_sigmoid)   xfc_gemm.cpp:17-40
  * with each 2-D tensor flattened to (pointer, rows, cols, stride0, stride1).

@@ -16,6 +16,7 @@ _vp, _i64, _f32, _sz, _int = C.c_void_p, C.c_int64, C.c_float, C.c_size_t, C.c_i
 _SIGNATURES = {
     "xfc_strerror": (C.c_char_p, [_int]),
     "xfc_abi_version": (_int, []),
+    "xfc_init": (_int, []),
     "xfc_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "xfc_gemm": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64,
                         _f32, _f32, _int, _vp, _sz, _vp]),

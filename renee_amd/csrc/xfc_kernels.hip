@@ -8,6 +8,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include <type_traits>
 
 #include "../../include/xfc_mi355x.h"
@@ -754,26 +756,41 @@ int check_launch() {
   return XFC_OK;
 }
 
-// Launch with `lds` bytes of dynamic LDS; sizes above the default limit need the attribute once per kernel.
-template <class K, class A>
-void launch_k(K kernel, dim3 g, dim3 b, int lds, hipStream_t st, const A& args) {
-  static bool raised = false;
-  if (!raised && lds > 48 * 1024) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    raised = true;
-  }
-  hipLaunchKernelGGL(kernel, g, b, lds, st, args);
+constexpr int MAX_DEVICES = 64;
+int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) dev = 0;
+  return dev;
+}
+
+// Dynamic LDS above the default limit needs the attribute once per kernel and device.
+template <auto Kernel>
+hipError_t raise_lds_limit(int lds) {
+  static std::atomic<bool> raised[MAX_DEVICES];
+  const int dev = current_device();
+  if (lds <= 48 * 1024 || raised[dev].load(std::memory_order_acquire)) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (e == hipSuccess) raised[dev].store(true, std::memory_order_release);
+  return e;
+}
+
+template <auto Kernel, class A>
+void launch_k(dim3 g, dim3 b, int lds, hipStream_t st, const A& args) {
+  raise_lds_limit<Kernel>(lds);
+  hipLaunchKernelGGL(Kernel, g, b, lds, st, args);
 }
 
 int num_cus() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
-    n = p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+  static std::atomic<int> n[MAX_DEVICES];
+  const int dev = current_device();
+  int v = n[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    int cnt = 0;
+    if (hipDeviceGetAttribute(&cnt, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cnt <= 0) cnt = 256;
+    v = cnt;
+    n[dev].store(v, std::memory_order_relaxed);
   }
-  return n;
+  return v;
 }
 
 constexpr size_t LOSS_PART_BYTES = 4096;  // one float per forward workgroup (at most 1024)
@@ -820,16 +837,16 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   if (grid > ids) grid = ids;                    // ids is a multiple of 8
   dim3 g((unsigned)grid), b(FwdCore::NT);
   if (mode == FWD_GRAD && loss_part) {
-    launch_k(fwd_kernel<FWD_GRAD, false, true>, g, b, FWD_LDS_BYTES, st, a);
+    launch_k<fwd_kernel<FWD_GRAD, false, true>>(g, b, FWD_LDS_BYTES, st, a);
     int rc = check_launch();
     if (rc) return rc;
     hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(64), 0, st, loss_part, (int)grid, loss_out);
     return check_launch();
   }
-  if (mode == FWD_GRAD) launch_k(fwd_kernel<FWD_GRAD, false>, g, b, FWD_LDS_BYTES, st, a);
-  else if (mode == FWD_SIGMOID && beta != 0.f) launch_k(fwd_kernel<FWD_SIGMOID, true>, g, b, FWD_LDS_BYTES, st, a);
-  else if (mode == FWD_SIGMOID) launch_k(fwd_kernel<FWD_SIGMOID, false>, g, b, FWD_LDS_BYTES, st, a);
-  else launch_k(fwd_kernel<FWD_LINEAR, false>, g, b, FWD_LDS_BYTES, st, a);
+  if (mode == FWD_GRAD) launch_k<fwd_kernel<FWD_GRAD, false>>(g, b, FWD_LDS_BYTES, st, a);
+  else if (mode == FWD_SIGMOID && beta != 0.f) launch_k<fwd_kernel<FWD_SIGMOID, true>>(g, b, FWD_LDS_BYTES, st, a);
+  else if (mode == FWD_SIGMOID) launch_k<fwd_kernel<FWD_SIGMOID, false>>(g, b, FWD_LDS_BYTES, st, a);
+  else launch_k<fwd_kernel<FWD_LINEAR, false>>(g, b, FWD_LDS_BYTES, st, a);
   return check_launch();
 }
 
@@ -858,7 +875,7 @@ int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float*
   a.M = M; a.N = N; a.K = K;
   const int64_t grid = (int64_t)a.tiles_m * a.tiles_n * a.splits;
   if (grid <= 0 || M <= 0 || N <= 0) return XFC_OK;
-  launch_k(dx_kernel, dim3((unsigned)grid), dim3(DxCore::NT), DX_LDS_BYTES, st, a);
+  launch_k<dx_kernel>(dim3((unsigned)grid), dim3(DxCore::NT), DX_LDS_BYTES, st, a);
   int rc = check_launch();
   if (rc) return rc;
   const int64_t nq = (int64_t)M * (N / 4);
@@ -876,8 +893,8 @@ int launch_dw(int mode, DwArgs a, hipStream_t st) {
   a.n_ids = (int)ids;
   int64_t grid = 2 * (int64_t)round_up(num_cus(), 8);  // two resident workgroups per CU
   if (grid > ids) grid = ids / 8 * 8 > 0 ? ids / 8 * 8 : ids;
-  if (mode == DW_UPDATE) launch_k(dw_kernel<DW_UPDATE>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
-  else launch_k(dw_kernel<DW_OUT>, dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  if (mode == DW_UPDATE) launch_k<dw_kernel<DW_UPDATE>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  else launch_k<dw_kernel<DW_OUT>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
   return check_launch();
 }
 
@@ -912,6 +929,26 @@ const char* xfc_strerror(int code) {
 }
 
 int xfc_abi_version(void) { return XFC_ABI_VERSION; }
+
+int xfc_init(void) {
+  hipError_t e = hipSuccess;
+  auto keep = [&](hipError_t r) { if (e == hipSuccess) e = r; };
+  keep(raise_lds_limit<fwd_kernel<FWD_GRAD, false, true>>(FWD_LDS_BYTES));
+  keep(raise_lds_limit<fwd_kernel<FWD_GRAD, false>>(FWD_LDS_BYTES));
+  keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID, true>>(FWD_LDS_BYTES));
+  keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID, false>>(FWD_LDS_BYTES));
+  keep(raise_lds_limit<fwd_kernel<FWD_LINEAR, false>>(FWD_LDS_BYTES));
+  keep(raise_lds_limit<dx_kernel>(DX_LDS_BYTES));
+  keep(raise_lds_limit<dw_kernel<DW_UPDATE>>(DW_LDS_BYTES));
+  keep(raise_lds_limit<dw_kernel<DW_OUT>>(DW_LDS_BYTES));
+  keep(raise_lds_limit<topk_kernel>(TOPK_LDS_BYTES));
+  (void)num_cus();
+  if (e != hipSuccess) {
+    fprintf(stderr, "xfc: xfc_init failed: %s\n", hipGetErrorString(e));
+    return XFC_ERR_HIP;
+  }
+  return XFC_OK;
+}
 
 size_t xfc_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (!dims_ok(M) || !dims_ok(N) || !dims_ok(K)) return 0;
@@ -1151,7 +1188,7 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   a.cand_v = reinterpret_cast<float*>(workspace);
   a.cand_i = reinterpret_cast<int32_t*>(a.cand_v + (size_t)a.n_groups * B * K);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  launch_k(topk_kernel, dim3((unsigned)grid), dim3(TopkCore::NT), TOPK_LDS_BYTES, st, a);
+  launch_k<topk_kernel>(dim3((unsigned)grid), dim3(TopkCore::NT), TOPK_LDS_BYTES, st, a);
   int rc = check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)B), dim3(64), 0, st, a.cand_v, a.cand_i, (int)B, a.n_groups, K,

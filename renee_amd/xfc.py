@@ -77,6 +77,54 @@ def xfc_gemm(mat_in1: torch.Tensor, mat_in2: torch.Tensor, mat_out: torch.Tensor
     check(rc, "xfc_gemm")
 
 
+def cosine_schedule_with_warmup(step: int, warmup_steps: int, total_steps: int, base_lr: float) -> float:
+    """Learning rate of the XFC optimizer at `step` (dl_base.py:241,376,396-397: transformers'
+    get_cosine_schedule_with_warmup, half a cosine period): linear from 0 over the warm-up, then
+    base_lr * 0.5 * (1 + cos(pi * progress)).  Pass the result as `lr=` to xfc_backward / dw_update."""
+    import math
+
+    if step < warmup_steps:
+        return base_lr * step / max(1, warmup_steps)
+    progress = (step - warmup_steps) / max(1, total_steps - warmup_steps)
+    return base_lr * max(0.0, 0.5 * (1.0 + math.cos(math.pi * progress)))
+
+
+def read_sparse_labels(path: str):
+    """Read a label matrix in the XC repository's sparse text format (header `rows cols`, then one line
+    per row of `col:val` pairs; the format main.py:50-51 loads through pyxclib) into CSR numpy arrays
+    (rowptr int64[rows+1], colidx int32[nnz], shape).  Values are ignored: labels are binary."""
+    import numpy as np
+
+    with open(path) as f:
+        rows, cols = (int(v) for v in f.readline().split()[:2])
+        rowptr = np.zeros(rows + 1, dtype=np.int64)
+        colidx = []
+        for r in range(rows):
+            toks = f.readline().split()
+            ids = sorted({int(t.split(":")[0]) for t in toks})
+            colidx.extend(ids)
+            rowptr[r + 1] = rowptr[r] + len(ids)
+    return rowptr, np.asarray(colidx, dtype=np.int32), (rows, cols)
+
+
+def batch_positives(rowptr, colidx, ids, start_label: int = 0, end_label: int | None = None):
+    """The collator's label tensor for a batch (dl_base.py:934-936: labels[full_ids].tocoo() as a
+    2 x nnz LongTensor, rows ascending), optionally restricted and re-based to one rank's label columns
+    (main.py:94-97)."""
+    import numpy as np
+
+    rows, cols = [], []
+    for b, i in enumerate(ids):
+        c = colidx[rowptr[i]:rowptr[i + 1]]
+        if end_label is not None:
+            c = c[(c >= start_label) & (c < end_label)]
+        elif start_label:
+            c = c[c >= start_label]
+        rows.append(np.full(c.shape[0], b, dtype=np.int64))
+        cols.append(c.astype(np.int64) - start_label)
+    return torch.from_numpy(np.stack([np.concatenate(rows), np.concatenate(cols)])) if rows else torch.zeros(2, 0, dtype=torch.int64)
+
+
 def coo_to_csr(pos_x: torch.Tensor, pos_y: torch.Tensor, num_rows: int):
     """Row-sorted COO (dl_base.py:934-936) -> (rowptr int32[B+1], colidx int32[nnz]) on the same device."""
     counts = torch.bincount(pos_x.long(), minlength=num_rows)
@@ -120,6 +168,8 @@ class XFCLayer:
         self.outsoft = torch.empty(self.max_batch, self.ldg, device=self.device, dtype=torch.float16)
         self.grad_input = torch.empty(self.max_batch, self.dims, device=self.device, dtype=torch.float32)
         self.xfc_weight_grad = None  # fp32 accumulator, only under split accumulation
+        with torch.cuda.device(self.device):
+            check(lib().xfc_init(), "xfc_init")
 
     # -- helpers ---------------------------------------------------------------------------
     def _x16(self, embed: torch.Tensor) -> torch.Tensor:
@@ -253,6 +303,29 @@ class XFCLayer:
                                         self.lr if lr is None else float(lr), self.momentum, self.weight_decay,
                                         _stream(self.xfc_weight))
         check(rc, "xfc_sgd_momentum")
+        self.xfc_weight_grad = None
+
+    # -- checkpoint payload (dl_base.py:412-446 keeps xfc_weight and the optimizer state per rank) ------
+    def state_dict(self) -> dict:
+        """W and the momentum as CPU fp16 tensors plus the hyper-parameters, for a checkpoint."""
+        return {"xfc_weight": self.xfc_weight.detach().cpu(), "momentum_buffer": self.momentum_buffer.detach().cpu(),
+                "numy": self.numy, "dims": self.dims, "lr": self.lr, "momentum": self.momentum,
+                "weight_decay": self.weight_decay}
+
+    def load_state_dict(self, state: dict) -> None:
+        """Restore from state_dict(); an fp32 xfc_weight (a reference checkpoint's) is rounded to fp16 once
+        and a missing momentum_buffer starts from zero, as the optimizer's first step does."""
+        w = state["xfc_weight"]
+        _require(tuple(w.shape) == (self.numy, self.dims), "checkpoint shape does not match this layer")
+        self.xfc_weight.copy_(w.to(device=self.device, dtype=torch.float16))
+        m = state.get("momentum_buffer")
+        if m is None:
+            self.momentum_buffer.zero_()
+        else:
+            self.momentum_buffer.copy_(m.to(device=self.device, dtype=torch.float16))
+        for k in ("lr", "momentum", "weight_decay"):
+            if k in state:
+                setattr(self, k, float(state[k]))
         self.xfc_weight_grad = None
 
     def xfc_backward(self, embed_out, pos_x, pos_y, grad_input=None, scale: float = 1.0,

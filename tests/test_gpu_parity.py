@@ -309,3 +309,21 @@ def test_fused_loss(dev, B, L, d):
     bce = float(torch.nn.BCEWithLogitsLoss(reduction="sum")(Z.double(), Y))
     assert abs(want - bce) <= 1e-6 * abs(bce)  # the oracle follows the reference and sums in float32
     assert abs(float(loss) - bce) <= 1e-5 * abs(bce)
+
+
+def test_state_dict_round_trip(dev):
+    B, L, d = 64, 1000, 64
+    X, W, P = _problem(B, L, d, seed=5)
+    px, py = P.coo()
+    a = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W)
+    a.xfc_backward(X.to(dev), px.to(dev), py.to(dev))
+    st = a.state_dict()
+    b = XFCLayer(L, d, B, dev, lr=0.01, momentum=0.5, seed=9)
+    b.load_state_dict(st)
+    a.xfc_backward(X.to(dev), px.to(dev), py.to(dev))
+    b.xfc_backward(X.to(dev), px.to(dev), py.to(dev))
+    assert torch.equal(a.xfc_weight, b.xfc_weight) and torch.equal(a.momentum_buffer, b.momentum_buffer)
+    # a reference checkpoint holds fp32 weights and may have no momentum yet
+    c = XFCLayer(L, d, B, dev, seed=1)
+    c.load_state_dict({"xfc_weight": W.float()})
+    assert torch.equal(c.xfc_weight.cpu(), W) and float(c.momentum_buffer.abs().sum()) == 0.0

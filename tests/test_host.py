@@ -109,3 +109,47 @@ def test_drop_in_module_name():
     import xfc_gemm_cuda  # dl_base.py:26-32, setup.py:8
 
     assert callable(xfc_gemm_cuda.xfc_gemm)
+
+
+def test_cosine_schedule_matches_closed_form():
+    import math
+
+    from renee_amd import cosine_schedule_with_warmup as sched
+
+    assert sched(0, 100, 1000, 0.05) == 0.0            # lr is 0 on the first step of a warm-up
+    assert abs(sched(50, 100, 1000, 0.05) - 0.025) < 1e-12
+    assert abs(sched(100, 100, 1000, 0.05) - 0.05) < 1e-12
+    assert abs(sched(550, 100, 1000, 0.05) - 0.025) < 1e-12
+    assert abs(sched(1000, 100, 1000, 0.05)) < 1e-12
+    for s in (101, 333, 999):
+        p = (s - 100) / 900
+        assert abs(sched(s, 100, 1000, 0.05) - 0.05 * 0.5 * (1 + math.cos(math.pi * p))) < 1e-15
+    try:
+        from transformers import get_cosine_schedule_with_warmup
+    except Exception:
+        return
+    prm = torch.nn.Parameter(torch.zeros(1))
+    opt = torch.optim.SGD([prm], lr=0.05)
+    sch = get_cosine_schedule_with_warmup(opt, 100, 1000)
+    for s in range(0, 1000, 37):
+        while sch.last_epoch < s:
+            opt.step()
+            sch.step()
+        assert abs(sch.get_last_lr()[0] - sched(s, 100, 1000, 0.05)) < 1e-12
+
+
+def test_sparse_label_reader_and_batch_positives():
+    from renee_amd import batch_positives, read_sparse_labels
+
+    path = os.path.join(ROOT, "tests", "golden", "lf_amazontitles_131k_tst_first256.txt")
+    rowptr, colidx, shape = read_sparse_labels(path)
+    assert shape == (256, 131073) and rowptr[-1] == len(colidx) and len(colidx) > 256
+    assert list(colidx[rowptr[0]:rowptr[1]]) == [42537, 43834]           # first row of the reference's file
+    assert list(colidx[rowptr[1]:rowptr[2]]) == [89490, 89491, 118419, 118424]
+    z = batch_positives(rowptr, colidx, [1, 0, 1])
+    assert z.dtype == torch.int64 and z.shape[0] == 2
+    assert z[0].tolist() == [0, 0, 0, 0, 1, 1, 2, 2, 2, 2]
+    assert z[1].tolist() == [89490, 89491, 118419, 118424, 42537, 43834, 89490, 89491, 118419, 118424]
+    # one rank's label columns, re-based (main.py:94-97)
+    zr = batch_positives(rowptr, colidx, [1, 0], start_label=65536, end_label=131088)
+    assert zr[0].tolist() == [0, 0, 0, 0] and zr[1].tolist() == [89490 - 65536, 89491 - 65536, 118419 - 65536, 118424 - 65536]
