@@ -60,9 +60,11 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// 16 bytes per lane from `g` to LDS at lds_base + lane*16 (lds_base wave-uniform).
+// 16 bytes per lane from `g` to LDS at lds_base + lane*16 (lds_base wave-uniform).  NT marks the
+// fetch non-temporal: for data read once, so that it does not displace reused lines from the L2.
+template <bool NT = false>
 __device__ __forceinline__ void load16_to_lds(const void* g, void* lds_base) {
-  __builtin_amdgcn_global_load_lds((XFC_GLB const void*)g, (XFC_LDS void*)lds_base, 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((XFC_GLB const void*)g, (XFC_LDS void*)lds_base, 16, 0, NT ? 2 : 0);
 }
 
 template <int BK>
@@ -76,7 +78,8 @@ __device__ __forceinline__ int kc_swz(int row) {
 // transposing read touches then sit in four different 64-byte bank groups.
 __device__ __forceinline__ int mc_swz(int k) { return (k & 3) << 2; }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_, bool ACC_AGPR_ = false>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_, bool ACC_AGPR_ = false,
+          bool A_NT_ = false, bool B_NT_ = false>
 struct PipeCore {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
@@ -112,7 +115,7 @@ struct PipeCore {
   // "uniform 64-bit base + per-thread 32-bit offset": the bases advance along k with scalar adds, so a
   // steady-state stage costs no vector ALU work, which matters because the SIMD that issues the MFMAs
   // cannot overlap them with other vector instructions.
-  template <bool KC, int R, int CH>
+  template <bool KC, int R, int CH, bool NT>
   struct Loader {
     static constexpr int CPI = KC ? CPR : R / 8;  // 16-byte chunks per tile row (KC) or per k-row (MC)
     static constexpr int RPI = 64 / CPI;          // tile rows (KC) or k-rows (MC) one wave instruction covers
@@ -160,20 +163,20 @@ struct PipeCore {
       if (k0 + BK <= kmax) {
 #pragma unroll
         for (int i = 0; i < CH; ++i)
-          load16_to_lds(base + grp[i] + kbytes + voff[i], region + (i * NW + wave) * 512);
+          load16_to_lds<NT>(base + grp[i] + kbytes + voff[i], region + (i * NW + wave) * 512);
       } else {  // the stage that crosses kmax: pieces past it come from the block of zeros
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
           const bool valid = k0 + kgrp[i] + kin < kmax;
           const void* src = valid ? (const void*)(base + grp[i] + kbytes + voff[i]) : (const void*)g_zero16;
-          load16_to_lds(src, region + (i * NW + wave) * 512);
+          load16_to_lds<NT>(src, region + (i * NW + wave) * 512);
         }
       }
       kbytes += kstep;
     }
   };
-  using LoaderA = Loader<A_KC, BM, A_CH>;
-  using LoaderB = Loader<B_KC, BN, B_CH>;
+  using LoaderA = Loader<A_KC, BM, A_CH, A_NT_>;
+  using LoaderB = Loader<B_KC, BN, B_CH, B_NT_>;
 
   __device__ __forceinline__ static half8 frag_kc(const half_t* lds, int row0, int kk, int lane) {
     const int r = row0 + (lane & 31);
