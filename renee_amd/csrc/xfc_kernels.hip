@@ -851,19 +851,27 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   return check_launch();
 }
 
-// Split count for dX: one workgroup per CU, a multiple of 8 slices (one slice of the label axis per
-// XCD at a time), each slice a multiple of the k-step.
+// Split count for dX: a multiple of 8 slices of the label axis (workgroup ids are dealt round-robin over
+// the 8 XCDs, so the tiles of one slice then meet in one L2), each slice a multiple of the k-step.  The
+// count minimises a cost model fitted to measurements: workgroups run in rounds of one per CU, every
+// workgroup pays a fixed prologue + partial-tile store, and the partial sums are written and read once.
 void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& k_per_split) {
   tiles_m = ceil_div(M, DxCore::BM);
   tiles_n = ceil_div(N, DxCore::BN);
-  const int tiles = tiles_m * tiles_n;
-  int s = num_cus() / (tiles > 0 ? tiles : 1);
-  s = s / 8 * 8;
-  if (s < 8) s = 8;
+  const int64_t tiles = (int64_t)tiles_m * tiles_n > 0 ? (int64_t)tiles_m * tiles_n : 1;
+  const int cus = num_cus();
+  const double nk = (double)ceil_div(K, DxCore::BK);
   const int max_s = (int)round_up(ceil_div(K, DxCore::BK), 8);
-  if (s > max_s) s = max_s;
-  k_per_split = (int)round_up(ceil_div(K, s), DxCore::BK);
-  splits = s;
+  constexpr double STAGE_US = 2.4, FIXED_STAGES = 6.0, PART_BYTES_PER_US = 3.0e6;
+  int best = 8;
+  double best_cost = 0.0;
+  for (int s = 8; s <= 256 && s <= max_s; s += 8) {
+    const double rounds = (double)ceil_div(tiles * s, cus);
+    const double cost = rounds * (nk / s + FIXED_STAGES) * STAGE_US + 2.0 * s * (double)M * N * 4.0 / PART_BYTES_PER_US;
+    if (s == 8 || cost < best_cost) { best = s; best_cost = cost; }
+  }
+  k_per_split = (int)round_up(ceil_div(K, best), DxCore::BK);
+  splits = best;
 }
 
 int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float* out, int64_t ldo, int M, int N, int K,
