@@ -159,14 +159,20 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* M, int6
                  void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Exact top-K labels per query row over all L labels, logits never written:
+ * Exact top-K labels per query row over all L labels:
  *   values[b][0..K-1], indices[b][0..K-1] = the K largest X[b].W[l], ties broken towards
  *   the lower label id.
  * Replaces FullPredictor's scoring loop, dl_base.py:736-756 (xfc_forward into outsoft,
- * then torch.max K times with the winners overwritten) and the pad clamp at
- * dl_base.py:782: indices >= numy are returned as numy-1.  1 <= K <= 8 <= L (the
- * reference's K > 5 branch, torch.topk at :756, is served by xfc_logits + a sort).
- * values are the fp32 accumulators (the reference returns the fp16-rounded logits).
+ * then torch.max K times with the winners overwritten, or torch.topk for K > 5) and the
+ * pad clamp at dl_base.py:782: indices >= numy are returned as numy-1.  1 <= K <= 128, K <= L.
+ *   K <= 8 (the reference's per-epoch K = 5): one fused pass, the logits are never
+ *     written; values are the fp32 accumulators (the reference returns fp16-rounded logits).
+ *   8 < K <= 128 (the reference's final evaluation, K = 100, dl_base.py:817-818): the fp16
+ *     logits of a block of rows go to the workspace and an exact selection kernel picks each
+ *     row's K largest; values are those fp16 logits widened to fp32, ties are between equal
+ *     fp16 values.  xfc_topk_workspace_bytes() asks for all B rows at once (B*round_up(L,8)*2
+ *     bytes); any 16-byte aligned workspace that holds min(B, 256) rows is accepted and the
+ *     rows are then processed in blocks of a multiple of 256.
  * Workspace: xfc_topk_workspace_bytes(B, L, K) bytes.
  */
 size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K);

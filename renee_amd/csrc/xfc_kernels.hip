@@ -477,6 +477,174 @@ __global__ void __launch_bounds__(64) topk_merge_kernel(const float* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------
+// top-K for 8 < K <= 128: exact selection over rows of fp16 logits (one workgroup per row)
+// ---------------------------------------------------------------------------------------------
+constexpr int SEL_MAX_K = 128;
+constexpr int SEL_THREADS = 1024;
+constexpr int SEL_BINS = 2048;  // histogram over the top 11 bits of the 16-bit key
+constexpr int SEL_CAP = 2048;   // candidates that are sorted in LDS
+
+// fp16 bit pattern -> 16-bit key that orders like the value (-0 counts as +0).
+__device__ __forceinline__ uint32_t sel_key(uint32_t h) {
+  if (h == 0x8000u) h = 0u;
+  return (h & 0x8000u) ? (~h & 0xffffu) : (h | 0x8000u);
+}
+__device__ __forceinline__ uint32_t sel_unkey(uint32_t k) { return (k & 0x8000u) ? (k & 0x7fffu) : (~k & 0xffffu); }
+
+struct SelLds {
+  int hist[SEL_BINS];
+  unsigned long long cand[SEL_CAP];
+  int wave_tot[SEL_THREADS / 64];
+  int n_cand, bin, above;
+};
+
+// The K largest of each row of `logits` (rows x L, leading dimension ldl, a multiple of 8), ordered by
+// (value descending, label ascending).  Pass 1 histograms the top 11 key bits and finds the bin that
+// holds the K-th largest; when at most SEL_CAP elements lie in that bin or above, they are gathered and
+// sorted.  Otherwise pass 2 histograms the bin's low 5 bits to get the exact K-th key; elements above it
+// are gathered, and the elements equal to it are taken in label order until K are found.
+__global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* __restrict__ logits, int64_t ldl, int L,
+                                                                   int64_t numy, int K, float* __restrict__ out_v,
+                                                                   int64_t* __restrict__ out_i) {
+  __shared__ SelLds S;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint16_t* row = reinterpret_cast<const uint16_t*>(logits) + (int64_t)blockIdx.x * ldl;
+  auto for_each = [&](auto&& f) {
+    for (int i = tid * 8; i < L; i += SEL_THREADS * 8) {
+      const uint4v q = *reinterpret_cast<const uint4v*>(row + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (i + e < L) f(sel_key((q[e >> 1] >> (16 * (e & 1))) & 0xffffu), i + e);
+    }
+  };
+  auto push = [&](uint32_t key, int idx) {
+    const int slot = atomicAdd(&S.n_cand, 1);
+    if (slot < SEL_CAP) S.cand[slot] = ((unsigned long long)(0xffffu - key) << 32) | (uint32_t)idx;
+  };
+  // Finds, over hist[0..nb), the highest bin b with (count in bins above b) + base < K <= that + hist[b];
+  // writes S.bin = b and S.above = base + count above b.  nb is a multiple of 64; executed by wave 0.
+  auto find_bin = [&](int nb, int base) {
+    if (wave == 0) {
+      const int per = nb / 64;
+      int p = 0;
+      for (int j = 0; j < per; ++j) p += S.hist[lane * per + j];
+      int suf = p;  // sum over lanes >= this one
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int v = __shfl_down(suf, off, 64);
+        if (lane + off < 64) suf += v;
+      }
+      const unsigned long long m = __ballot(base + suf >= K);
+      const int owner = 63 - __builtin_clzll(m | 1ull);  // m != 0 because K <= L
+      if (lane == owner) {
+        int above = base + suf - p, b = lane * per + per - 1;
+        for (; b > lane * per; --b) {
+          if (above + S.hist[b] >= K) break;
+          above += S.hist[b];
+        }
+        S.bin = b;
+        S.above = above;
+      }
+    }
+  };
+
+  for (int b = tid; b < SEL_BINS; b += SEL_THREADS) S.hist[b] = 0;
+  if (tid == 0) S.n_cand = 0;
+  __syncthreads();
+  for_each([&](uint32_t key, int) { atomicAdd(&S.hist[key >> 5], 1); });
+  __syncthreads();
+  find_bin(SEL_BINS, 0);
+  __syncthreads();
+  const int bin = S.bin, above = S.above;
+  const int in_bin = S.hist[bin];
+  __syncthreads();
+  if (above + in_bin <= SEL_CAP) {
+    for_each([&](uint32_t key, int idx) { if ((int)(key >> 5) >= bin) push(key, idx); });
+  } else {
+    if (tid < 64) S.hist[tid] = 0;
+    __syncthreads();
+    for_each([&](uint32_t key, int) { if ((int)(key >> 5) == bin) atomicAdd(&S.hist[key & 31u], 1); });
+    __syncthreads();
+    find_bin(64, above);
+    __syncthreads();
+    const uint32_t thr = ((uint32_t)bin << 5) | (uint32_t)S.bin;
+    const int n_gt = S.above, n_eq = S.hist[S.bin];
+    __syncthreads();
+    if (n_gt + n_eq <= SEL_CAP) {
+      for_each([&](uint32_t key, int idx) { if (key >= thr) push(key, idx); });
+    } else {
+      // too many copies of the K-th value to sort: those above it first, then its copies in label order
+      for_each([&](uint32_t key, int idx) { if (key > thr) push(key, idx); });
+      const int need = K - n_gt;
+      int taken = 0;
+      for (int base = 0; base < L && taken < need; base += SEL_THREADS * 8) {
+        const int i = base + tid * 8;
+        uint32_t hit = 0;
+        if (i < L) {
+          const uint4v q = *reinterpret_cast<const uint4v*>(row + i);
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (i + e < L && sel_key((q[e >> 1] >> (16 * (e & 1))) & 0xffffu) == thr) hit |= 1u << e;
+        }
+        const int c = __builtin_popcount(hit);
+        int inc = c;  // inclusive scan over the wave
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const int v = __shfl_up(inc, off, 64);
+          if (lane >= off) inc += v;
+        }
+        if (lane == 63) S.wave_tot[wave] = inc;
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int w = 0; w < SEL_THREADS / 64; ++w) {
+          const int t = S.wave_tot[w];
+          if (w < wave) before += t;
+          total += t;
+        }
+        int rank = taken + before + inc - c;
+        for (int e = 0; e < 8; ++e)
+          if (hit & (1u << e)) {
+            if (rank < need) S.cand[n_gt + rank] = ((unsigned long long)(0xffffu - thr) << 32) | (uint32_t)(i + e);
+            ++rank;
+          }
+        taken += total;
+        __syncthreads();
+      }
+      if (tid == 0) S.n_cand = K;
+    }
+  }
+  __syncthreads();
+  const int n = S.n_cand;  // K <= n <= SEL_CAP
+  int n2 = 1;
+  while (n2 < n) n2 <<= 1;
+  for (int i = n + tid; i < n2; i += SEL_THREADS) S.cand[i] = ~0ull;
+  __syncthreads();
+  for (int k = 2; k <= n2; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int i = tid; i < n2; i += SEL_THREADS) {
+        const int x = i ^ j;
+        if (x > i) {
+          const unsigned long long a = S.cand[i], b = S.cand[x];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) { S.cand[i] = b; S.cand[x] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  if (tid < K) {
+    const unsigned long long c = S.cand[tid];
+    const uint32_t hbits = sel_unkey(0xffffu - (uint32_t)(c >> 32));
+    const uint16_t h16 = (uint16_t)hbits;
+    half_t h;
+    __builtin_memcpy(&h, &h16, 2);
+    int64_t idx = (int64_t)(uint32_t)c;
+    if (idx >= numy) idx = numy - 1;
+    out_v[(int64_t)blockIdx.x * K + tid] = (float)h;
+    out_i[(int64_t)blockIdx.x * K + tid] = idx;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
 using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, true>;  // accumulators in AGPRs
@@ -1174,7 +1342,8 @@ static void topk_plan(int64_t B, int64_t L, int& tiles_m, int& tiles_n, int& n_g
 }
 
 size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K) {
-  if (!dims_ok(B) || !dims_ok(L) || K < 1 || K > TOPK_MAX || B == 0 || L == 0) return 0;
+  if (!dims_ok(B) || !dims_ok(L) || K < 1 || K > SEL_MAX_K || B == 0 || L == 0) return 0;
+  if (K > TOPK_MAX) return (size_t)B * (size_t)round_up(L, 8) * 2;  // the logits of every row
   int tm, tn, ng, grid;
   topk_plan(B, L, tm, tn, ng, grid);
   return (size_t)ng * B * K * 8;
@@ -1184,9 +1353,29 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
              int K, float* values, int64_t* indices, void* workspace, size_t workspace_bytes, void* stream) {
   if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
   if (B == 0) return XFC_OK;
-  if (K < 1 || K > TOPK_MAX || L < K || numy < 1 || d <= 0) return XFC_ERR_INVALID;
+  if (K < 1 || K > SEL_MAX_K || L < K || numy < 1 || d <= 0) return XFC_ERR_INVALID;
   if (!X || !W || !values || !indices) return XFC_ERR_INVALID;
   if (ldx % 8 || ldw % 8 || d % 8 || !aligned16(X) || !aligned16(W)) return XFC_ERR_ALIGN;
+  if (K > TOPK_MAX) {
+    // logits of a block of rows into the workspace, then an exact selection per row
+    const int64_t ldl = round_up(L, 8);
+    const int64_t fit = workspace ? (int64_t)(workspace_bytes / (size_t)(ldl * 2)) : 0;
+    if (fit < (B < 256 ? B : 256)) return XFC_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return XFC_ERR_ALIGN;
+    const int64_t block = fit >= B ? B : fit / 256 * 256;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    for (int64_t r0 = 0; r0 < B; r0 += block) {
+      const int64_t rows = B - r0 < block ? B - r0 : block;
+      int rc = launch_fwd(FWD_LINEAR, (const half_t*)X + r0 * ldx, ldx, (const half_t*)W, ldw, (half_t*)workspace, ldl,
+                          (int)rows, (int)L, (int)d, (int)L, 1.0f, 0.0f, nullptr, st);
+      if (rc) return rc;
+      hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)rows), dim3(SEL_THREADS), 0, st, (const half_t*)workspace,
+                         ldl, (int)L, numy, K, values + r0 * K, indices + r0 * K);
+      rc = check_launch();
+      if (rc) return rc;
+    }
+    return XFC_OK;
+  }
   TopkArgs a;
   int grid;
   topk_plan(B, L, a.tiles_m, a.tiles_n, a.n_groups, grid);

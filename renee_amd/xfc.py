@@ -196,18 +196,25 @@ class XFCLayer:
         check(rc, "xfc_logits")
         return out
 
-    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None):
+    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None,
+             max_workspace_bytes: int = 8 << 30):
         """Exact top-K labels per row over all labels (FullPredictor's scoring loop, dl_base.py:736-756,
         with the pad clamp of :782 when numy < the stored label count).  Returns (values fp32, indices
-        int64), each (batch, K); ties go to the lower label id.  K <= 8."""
+        int64), each (batch, K); ties go to the lower label id.  K <= 128: up to 8 in one fused pass,
+        above that (the final evaluation's K = 100, dl_base.py:817-818) by an exact selection over fp16
+        logits held in the workspace, at most `max_workspace_bytes` of them at a time."""
         x = self._x16(embed)
         bsz = x.shape[0]
-        _require(1 <= K <= 8, "K must be in 1..8 (for larger K take xfc_forward and sort)")
+        _require(1 <= K <= 128 and K <= self.numy, "K must be in 1..min(128, numy)")
         vals = torch.empty(bsz, K, device=self.device, dtype=torch.float32)
         inds = torch.empty(bsz, K, device=self.device, dtype=torch.int64)
         L = lib()
         with torch.cuda.device(self.device):
-            ws = _workspace.get(self.device, L.xfc_topk_workspace_bytes(bsz, self.numy, K))
+            need = L.xfc_topk_workspace_bytes(bsz, self.numy, K)
+            if K > 8 and need > max_workspace_bytes:  # rows in blocks of a multiple of 256
+                row_bytes = self.ldg * 2
+                need = max(256, max_workspace_bytes // row_bytes // 256 * 256) * row_bytes
+            ws = _workspace.get(self.device, need)
             rc = L.xfc_topk(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims, bsz, self.numy,
                             self.dims, self.numy if numy is None else int(numy), int(K), vals.data_ptr(),
                             inds.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))

@@ -96,6 +96,21 @@ def test_config3_ragged_labels_and_top5(dev):
             gap = min(abs(float(best_v[b, j] - other)), abs(float(best_v[b, max(j - 1, 0)] - best_v[b, j])) or 1e9)
             assert gap <= 1e-5 * scale, (b, j)
     assert float(mism.float().mean()) < 0.01
+    # the final evaluation's K = 100 (dl_base.py:817-818) at the same size: against torch.topk of the same
+    # fp16 logits (values exact; indices must point at those values, ascending within equal values)
+    torch.cuda.synchronize()
+    print("top-100 at configs[3] size", flush=True)
+    v100, i100 = lay.topk(X, 100)
+    Zg = lay.xfc_forward(X)
+    tv, _ = torch.topk(Zg, 100, dim=1)
+    assert torch.equal(v100, tv.float())
+    assert torch.equal(torch.gather(Zg, 1, i100).float(), v100)
+    same = v100[:, 1:] == v100[:, :-1]
+    assert bool((i100[:, 1:] > i100[:, :-1])[same].all())
+    srt, _ = torch.sort(i100, dim=1)
+    assert bool((srt[:, 1:] != srt[:, :-1]).all())
+    # the fused K = 5 scorer and the selection agree on the leaders (fp16 rounding can swap near-equal ones)
+    assert float((i100[:, :5] == i).float().mean()) > 0.95
 
 
 def test_config4_streaming_shape(dev):

@@ -88,3 +88,101 @@ def test_topk_rising_scores_exact_rescan(dev):
     X = (X.float() * 0 + base.unsqueeze(0) + 0.05 * synth.make_X(B, d, 5)).half()
     _check(dev, X, W, 5)
     _check(dev, X, W, 8)
+
+
+# ---- 8 < K <= 128: exact selection over fp16 logits (the final evaluation's K = 100, dl_base.py:817-818) ----
+def _check_select(dev, X, W, K, numy=None, max_ws=None, vs_oracle=True):
+    B, d = X.shape
+    L = W.shape[0]
+    lay = XFCLayer(L, d, B, dev, weight=W)
+    print(f"topk-select: B={B} L={L} d={d} K={K} numy={numy} max_ws={max_ws}", flush=True)
+    kw = {} if max_ws is None else {"max_workspace_bytes": max_ws}
+    v, i = lay.topk(X.to(dev), K, numy, **kw)
+    v, i = v.cpu(), i.cpu()
+    # (a) the selection itself, against a stable sort of the same fp16 logits: exact
+    Zg = lay.xfc_forward(X.to(dev)).float().cpu()
+    sv, si = torch.sort(Zg, dim=1, descending=True, stable=True)
+    ev, ei = sv[:, :K], si[:, :K]
+    if numy is not None:
+        ei = torch.where(ei >= numy, torch.full_like(ei, numy - 1), ei)
+    assert torch.equal(v, ev)
+    assert torch.equal(i, ei)
+    if not vs_oracle:
+        return i
+    # (b) against the oracle's fp32 scores: values to fp16 rounding, indices except between near-equal scores
+    Z = O.logits(X.float(), W.float())
+    ov, oi = torch.sort(Z, dim=1, descending=True, stable=True)
+    scale = float(Z.abs().max())
+    assert torch.allclose(v, ov[:, :K], rtol=0, atol=1e-3 * scale)
+    near = 1.5e-3 * scale
+    kth = ov[:, K - 1]
+    chosen = torch.gather(Z, 1, si[:, :K])
+    assert bool((chosen >= kth[:, None] - near).all())          # nothing clearly below the K-th was taken
+    must = Z > (kth[:, None] + near)                            # everything clearly above it was
+    took = torch.zeros_like(must)
+    took.scatter_(1, si[:, :K], True)
+    assert bool((took | ~must).all())
+    return i
+
+
+@pytest.mark.parametrize("B,L,d,K", [(37, 1000, 64, 100), (256, 4096, 768, 100), (64, 70001, 128, 9),
+                                     (5, 128, 8, 128), (3, 100, 8, 100)])
+def test_topk_select_matches_sort_and_oracle(dev, B, L, d, K):
+    X = synth.make_X(B, d, 4).half()
+    W = synth.make_W(L, d, 4).half()
+    _check_select(dev, X, W, K)
+
+
+def test_topk_select_row_blocks_and_pad_clamp(dev):
+    """A workspace smaller than all rows' logits: rows go in blocks of 256 (600 -> 256 + 256 + 88)."""
+    B, L, d = 600, 3001, 64
+    X = synth.make_X(B, d, 5).half()
+    W = synth.make_W(L, d, 5).half()
+    i = _check_select(dev, X, W, 100, numy=2990, max_ws=300 * 3008 * 2)
+    assert int(i.max()) <= 2989
+
+
+def _axis_problem(scores, B=3):
+    """Logits that are exactly the given fp16 numbers: X rows are multiples of e_0, W[:, 0] = scores."""
+    L = scores.numel()
+    X = torch.zeros(B, 8, dtype=torch.float16)
+    X[:, 0] = torch.tensor([1.0, 2.0, 0.5][:B], dtype=torch.float16)
+    W = torch.zeros(L, 8, dtype=torch.float16)
+    W[:, 0] = scores
+    return X, W
+
+
+def test_topk_select_crowded_bin_takes_the_refining_pass(dev):
+    """4000 labels whose scores are the 32 fp16 numbers of one histogram bin [1, 1+32/1024): more than the
+    sort capacity lie in the K-th value's bin, so its low key bits are histogrammed as well."""
+    g = torch.Generator().manual_seed(6)
+    L = 6000
+    scores = (torch.rand(L, generator=g) * 0.5).half()
+    crowd = torch.randperm(L, generator=g)[:4000]
+    scores[crowd] = (1.0 + torch.randint(0, 32, (4000,), generator=g).float() / 1024).half()
+    X, W = _axis_problem(scores)
+    _check_select(dev, X, W, 100, vs_oracle=False)
+    _check_select(dev, X, W, 128, vs_oracle=False)
+
+
+def test_topk_select_many_copies_of_the_kth_value(dev):
+    """3000 labels share the K-th largest score (more than can be sorted): they are taken in label order;
+    also a constant row, signed zeros and negative scores."""
+    g = torch.Generator().manual_seed(7)
+    L = 9000
+    scores = (torch.rand(L, generator=g) * 0.5 - 1.0).half()      # negative background
+    same = torch.randperm(L, generator=g)[:3000]
+    scores[same] = 0.75
+    top = torch.randperm(L, generator=g)[:40]
+    scores[top] = (1.0 + torch.arange(40).float() / 64).half()    # 40 distinct larger scores (some overwrite 0.75)
+    X, W = _axis_problem(scores)
+    i = _check_select(dev, X, W, 100, vs_oracle=False)
+    ties = sorted(set(same.tolist()) - set(top.tolist()))
+    assert i[0, 40:].tolist() == ties[:60]
+    # every logit equal (zero weights): the first K labels, in order; -0 and +0 are one value
+    Wz = torch.zeros(L, 8, dtype=torch.float16)
+    Xz = torch.zeros(2, 8, dtype=torch.float16)
+    Xz[0, 0], Xz[1, 0] = 1.0, -1.0
+    Wz[::2, 0] = -0.0
+    iz = _check_select(dev, Xz, Wz, 100, vs_oracle=False)
+    assert iz[0].tolist() == list(range(100)) and iz[1].tolist() == list(range(100))
