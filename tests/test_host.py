@@ -153,3 +153,35 @@ def test_sparse_label_reader_and_batch_positives():
     # one rank's label columns, re-based (main.py:94-97)
     zr = batch_positives(rowptr, colidx, [1, 0], start_label=65536, end_label=131088)
     assert zr[0].tolist() == [0, 0, 0, 0] and zr[1].tolist() == [89490 - 65536, 89491 - 65536, 118419 - 65536, 118424 - 65536]
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """include/xfc_mi355x.h must be usable from C (the boundary a cgo / JNI / ctypes binding sees): it
+    compiles as C99 and a C program linked against the library can call the argument checks."""
+    import shutil
+    import subprocess
+
+    from renee_amd._lib import LIB_PATH
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    hdr = os.path.join(ROOT, "include", "xfc_mi355x.h")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", hdr],
+                   check=True)
+    if not os.path.exists(LIB_PATH):
+        pytest.skip("library not built")
+    src = tmp_path / "t.c"
+    src.write_text('#include <stdio.h>\n#include "xfc_mi355x.h"\n'
+                   'int main(void) {\n'
+                   '  if (xfc_abi_version() != XFC_ABI_VERSION) return 1;\n'
+                   '  if (xfc_logits(NULL, 8, NULL, 8, NULL, 8, 4, 4, 8, NULL) != XFC_ERR_INVALID) return 2;\n'
+                   '  if (xfc_topk_workspace_bytes(4, 1000, 129) != 0) return 3;\n'
+                   '  if (xfc_topk_workspace_bytes(4, 1000, 100) != (size_t)4 * 1000 * 2) return 4;\n'
+                   '  printf("%s\\n", xfc_strerror(XFC_ERR_WORKSPACE));\n  return 0;\n}\n')
+    exe = tmp_path / "t"
+    libdir = os.path.dirname(LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                    "-L", libdir, "-l:" + os.path.basename(LIB_PATH), "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out
+    assert "workspace" in out.stdout.lower()
