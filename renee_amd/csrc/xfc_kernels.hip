@@ -945,7 +945,8 @@ hipError_t raise_lds_limit(int lds) {
 
 template <auto Kernel, class A>
 void launch_k(dim3 g, dim3 b, int lds, hipStream_t st, const A& args) {
-  raise_lds_limit<Kernel>(lds);
+  // a failure stays recorded as the runtime's last error, which check_launch() reports
+  if (raise_lds_limit<Kernel>(lds) != hipSuccess) return;
   hipLaunchKernelGGL(Kernel, g, b, lds, st, args);
 }
 
