@@ -327,3 +327,28 @@ def test_state_dict_round_trip(dev):
     c = XFCLayer(L, d, B, dev, seed=1)
     c.load_state_dict({"xfc_weight": W.float()})
     assert torch.equal(c.xfc_weight.cpu(), W) and float(c.momentum_buffer.abs().sum()) == 0.0
+
+
+def test_seeded_shape_sweep(dev):
+    """Sixteen seeded shapes off every tile boundary (batch 1..520, labels 8..6000, d a multiple of 8 up
+    to 384), X handed over as a strided view, random weight decay and loss scale: one whole step each."""
+    rng = np.random.default_rng(123)
+    for case in range(16):
+        B = int(rng.integers(1, 521))
+        L = int(rng.integers(8, 6001))
+        d = 8 * int(rng.integers(1, 49))
+        wd = float(rng.choice([0.0, 1e-4, 1e-2]))
+        scale = float(rng.choice([1.0, 4096.0, 0.5]))
+        X, W, P = _problem(B, L, d, kmax=min(8, L), seed=1000 + case)
+        px, py = P.coo()
+        wide = torch.zeros(B, d + 8 * int(rng.integers(0, 3)), dtype=torch.float16)
+        wide[:, :d] = X
+        print(f"sweep case {case}: B={B} L={L} d={d} ld={wide.shape[1]} wd={wd} scale={scale}", flush=True)
+        lay = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=wd, weight=W)
+        Xd = wide.to(dev)[:, :d]
+        ref = O.step(X.float(), W.float(), torch.zeros(L, d), px, py, 0.05, 0.9, wd, scale)
+        dX = lay.xfc_backward(Xd, px.to(dev), py.to(dev), scale=scale)
+        assert rel(lay.outsoft[:B, :L], ref["G"]) <= TOL
+        assert rel(dX[:B], ref["dX"]) <= TOL
+        assert rel(lay.xfc_weight, ref["W"]) <= TOL
+        assert rel(lay.momentum_buffer, ref["M"]) <= TOL
