@@ -7,7 +7,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 
-from .build import LIB_PATH
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libxfc_mi355x.so")  # written by renee_amd/build.py
 
 _lib = None
 
