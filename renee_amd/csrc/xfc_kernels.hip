@@ -102,7 +102,7 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
 // ---------------------------------------------------------------------------------------------
 // forward: out = epilogue(alpha * X . W^T + beta * out)
 // ---------------------------------------------------------------------------------------------
-enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2 };
+enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2, FWD_SIGMOID_PLAIN = 3 };  // PLAIN: alpha 1, beta 0
 
 using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true>;
 // beside the ring: the tile's positives bitmap, later reused as store staging (8 rows x TN labels per wave)
@@ -1015,6 +1015,7 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   }
   if (mode == FWD_GRAD) launch_k<fwd_kernel<FWD_GRAD, false>>(g, b, FWD_LDS_BYTES, st, a);
   else if (mode == FWD_SIGMOID && beta != 0.f) launch_k<fwd_kernel<FWD_SIGMOID, true>>(g, b, FWD_LDS_BYTES, st, a);
+  else if (mode == FWD_SIGMOID && alpha == 1.0f) launch_k<fwd_kernel<FWD_SIGMOID_PLAIN, false>>(g, b, FWD_LDS_BYTES, st, a);
   else if (mode == FWD_SIGMOID) launch_k<fwd_kernel<FWD_SIGMOID, false>>(g, b, FWD_LDS_BYTES, st, a);
   else launch_k<fwd_kernel<FWD_LINEAR, false>>(g, b, FWD_LDS_BYTES, st, a);
   return check_launch();
@@ -1115,6 +1116,7 @@ int xfc_init(void) {
   keep(raise_lds_limit<fwd_kernel<FWD_GRAD, false>>(FWD_LDS_BYTES));
   keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID, true>>(FWD_LDS_BYTES));
   keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID, false>>(FWD_LDS_BYTES));
+  keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID_PLAIN, false>>(FWD_LDS_BYTES));
   keep(raise_lds_limit<fwd_kernel<FWD_LINEAR, false>>(FWD_LDS_BYTES));
   keep(raise_lds_limit<dx_kernel>(DX_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_UPDATE>>(DW_LDS_BYTES));
