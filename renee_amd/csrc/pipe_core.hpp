@@ -60,11 +60,39 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// 16 bytes per lane from `g` to LDS at lds_base + lane*16 (lds_base wave-uniform).  NT marks the
-// fetch non-temporal: for data read once, so that it does not displace reused lines from the L2.
+// 16 bytes per lane from global memory to LDS at lds_base + lane*16 (lds_base wave-uniform), as
+// global_load_lds_dwordx4 with the LDS address in M0.  Written as inline asm on purpose: the compiler
+// treats the builtin form as a store to LDS that any later LDS read it cannot disambiguate may alias, and
+// puts an s_waitcnt vmcnt(0) in front of such reads (every ds_read_b64_tr_b16 and every epilogue access to
+// LDS), which makes each wave wait for the stage it has just requested.  The waits for these fetches are
+// the explicit ones in run(); the compiler's own vmcnt bookkeeping for other loads and stores stays
+// correct without knowing about them (operations return in order, so it can only wait longer than
+// needed).  NT marks the fetch non-temporal: for data read once, so that it does not displace reused
+// lines from the L2.
+__device__ __forceinline__ uint32_t lds_addr(void* p) { return (uint32_t)(uintptr_t)(XFC_LDS void*)p; }
+// address = uniform 64-bit base + per-lane 32-bit offset
+template <bool NT = false>
+__device__ __forceinline__ void load16_to_lds(const void* ubase, uint32_t voff, void* lds_base) {
+  const uint32_t m = lds_addr(lds_base);
+  // an integer operand whose halves are marked uniform: the "s" constraint alone is not always honoured
+  const uint64_t b0 = reinterpret_cast<uint64_t>(ubase);
+  // (readfirstlane returns a signed int: widen through uint32_t, or the low half sign-extends into the high one)
+  const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b0 >> 32));
+  const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b0);
+  const uint64_t b = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+  if constexpr (NT)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m), "v"(voff), "s"(b) : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(voff), "s"(b) : "memory");
+}
+// address = per-lane 64-bit pointer
 template <bool NT = false>
 __device__ __forceinline__ void load16_to_lds(const void* g, void* lds_base) {
-  __builtin_amdgcn_global_load_lds((XFC_GLB const void*)g, (XFC_LDS void*)lds_base, 16, 0, NT ? 2 : 0);
+  const uint32_t m = lds_addr(lds_base);
+  if constexpr (NT)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(m), "v"(g) : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m), "v"(g) : "memory");
 }
 
 template <int BK>
@@ -163,7 +191,7 @@ struct PipeCore {
       if (k0 + BK <= kmax) {
 #pragma unroll
         for (int i = 0; i < CH; ++i)
-          load16_to_lds<NT>(base + grp[i] + kbytes + voff[i], region + (i * NW + wave) * 512);
+          load16_to_lds<NT>(base + grp[i] + kbytes, voff[i], region + (i * NW + wave) * 512);
       } else {  // the stage that crosses kmax: pieces past it come from the block of zeros
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
@@ -311,7 +339,7 @@ struct PipeCore {
       } else {
         // past the last stage: keep the count of outstanding fetches per iteration constant
 #pragma unroll
-        for (int i = 0; i < LOADS_PER_STAGE; ++i) load16_to_lds((const void*)g_zero16, st + (i * NW + wave) * 512);
+        for (int i = 0; i < LOADS_PER_STAGE; ++i) load16_to_lds((const void*)g_zero16, 0u, st + (i * NW + wave) * 512);
       }
       i_slot = i_slot + 1 == STAGES ? 0 : i_slot + 1;
     };
