@@ -728,7 +728,7 @@ __global__ void __launch_bounds__(256) dx_reduce_kernel(const float* __restrict_
 // ---------------------------------------------------------------------------------------------
 enum DwMode { DW_OUT = 0, DW_UPDATE = 1 };
 
-using DwCore = PipeCore<128, 256, 32, 2, 2, 3, false, false>;
+using DwCore = PipeCore<128, 256, 32, 2, 2, 2, false, false>;
 constexpr int DW_STAGE_FLOATS = 8 * 64;  // per wave: 8 label rows x 64 dims
 constexpr int DW_LDS_BYTES = DwCore::LDS_BYTES + DwCore::NW * DW_STAGE_FLOATS * 4;
 static_assert(DwCore::FN % 2 == 0, "epilogue walks pairs of 32-column blocks");
@@ -782,12 +782,14 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
     auto strip_row = [&](int s) { return m0 + wm * C::TM + (s / (4 * (C::FN / 2))) * 32 + 8 * ((s / (C::FN / 2)) % 4) + srow; };
     auto strip_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 8; };
     half8 wq[DEPTH], mq[DEPTH];
+    // unconditional (out-of-range strips read the last valid row / column block and are not stored):
+    // straight-line loads let the compiler count exactly how many may stay in flight at each use
     auto fetch = [&](int s, half8& wv, half8& mv) {
-      const int row = strip_row(s), col = strip_col(s);
-      if (row < a.M && col < a.N) {
-        wv = __builtin_nontemporal_load(reinterpret_cast<const half8*>(a.Wt + (int64_t)row * a.ldw + col));
-        mv = __builtin_nontemporal_load(reinterpret_cast<const half8*>(a.Mo + (int64_t)row * a.ldm + col));
-      }
+      int row = strip_row(s), col = strip_col(s);
+      row = row < a.M ? row : a.M - 1;
+      col = col < a.N ? col : a.N - 8;
+      wv = __builtin_nontemporal_load(reinterpret_cast<const half8*>(a.Wt + (int64_t)row * a.ldw + col));
+      mv = __builtin_nontemporal_load(reinterpret_cast<const half8*>(a.Mo + (int64_t)row * a.ldm + col));
     };
     if constexpr (MODE == DW_UPDATE) {
 #pragma unroll
