@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
 # HBM bytes per launch of the dW+update kernel at configs[2]: rocprofv3 --pmc FETCH_SIZE (2,860,723.5 KiB,
 # x2.000 from the 1 GiB copy) + WRITE_SIZE (3,932,160 KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
-DW_UPDATE_TRAFFIC_BYTES = {2: (2 * 2808059.7 + 3932160.0) * 1024.0}
+DW_UPDATE_TRAFFIC_BYTES = {2: (2 * 2820425.4 + 3932160.0) * 1024.0}
 
 
 def cpu_baseline(cfg: int, d: int, seed: int):
