@@ -20,8 +20,11 @@ namespace xfc {
 // ---------------------------------------------------------------------------------------------
 // helpers
 // ---------------------------------------------------------------------------------------------
+// 1 / (1 + 2^(-z log2 e)) with the bare v_exp_f32 / v_rcp_f32: the exponential may flush to zero or
+// overflow to infinity at the ends, where the quotient is 1 or 0 either way, so the range fix-up that
+// __expf carries (a compare and a select per element) buys nothing here.
 __device__ __forceinline__ float sigmoidf_fast(float z) {
-  return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.44269504088896341f));
 }
 
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Tiles that
@@ -135,7 +138,7 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
   uint32_t* bm = reinterpret_cast<uint32_t*>(smem_raw + C::LDS_BYTES);
   const int G = gridDim.x, w = blockIdx.x;
   const int n_items = (a.n_ids - w + G - 1) / G;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and known to be
   const int wm = wave / C::WN, wn = wave % C::WN;
   half_t* stg = reinterpret_cast<half_t*>(bm) + wave * FWD_STG_HALVES;  // 8 rows x TN labels
   float loss_acc = 0.f;  // LOSS: this lane's share of sum softplus(z) - sum z[positives]
@@ -185,6 +188,9 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
     // The per-element work below is the vector ALU cost of the whole tile (the SIMD cannot overlap it
     // with MFMAs), so the rare cases -- a tile holding positives, a tile crossing the label count -- are
     // compiled as separate paths and the common one carries neither.
+    int64_t lane_off[C::FN / 2];  // where this lane's 16 bytes of a staged strip go, relative to the strip
+#pragma unroll
+    for (int p = 0; p < C::FN / 2; ++p) lane_off[p] = (int64_t)((lane + 64 * p) / CHS) * a.ldo + ((lane + 64 * p) % CHS) * 8;
     auto body = [&](auto pos_tag, auto edge_tag) {
       constexpr bool POS = decltype(pos_tag)::value, EDGE = decltype(edge_tag)::value;
       float tile_loss = 0.f;
@@ -233,7 +239,8 @@ __global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
             const int row = m0 + wm * C::TM + fm * 32 + 8 * q + srow;
             const int col = n0 + wn * C::TN + sch * 8;
             if (row < a.M) {
-              half_t* dst = a.out + (int64_t)row * a.ldo + col;
+              // uniform part + per-lane part computed once per tile: no per-strip vector multiply
+              half_t* dst = a.out + ((int64_t)(m0 + wm * C::TM + fm * 32 + 8 * q) * a.ldo + n0 + wn * C::TN) + lane_off[p];
               if (!EDGE || col + 8 <= a.n_store) {
                 __builtin_nontemporal_store(v8, reinterpret_cast<half8*>(dst));  // G is not re-read before it leaves the L2
               } else {
@@ -346,7 +353,7 @@ __global__ void __launch_bounds__(TopkCore::NT) topk_kernel(TopkArgs a) {
   int mt, grp;
   xcd_map(blockIdx.x, a.tiles_m, mt, grp);
   const int n_items = grp < a.tiles_n ? (a.tiles_n - grp + a.n_groups - 1) / a.n_groups : 0;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and known to be
   const int wm = wave / C::WN, wn = wave % C::WN;
   const int m0 = mt * C::BM;
   const int K = a.topk;
@@ -670,7 +677,7 @@ __global__ void __launch_bounds__(DxCore::NT) dx_kernel(DxArgs a) {
   const int64_t kb64 = (int64_t)split * a.k_per_split;
   const int k_begin = (int)(kb64 < a.K ? kb64 : a.K);
   const int k_end = (int)(kb64 + a.k_per_split < a.K ? kb64 + a.k_per_split : a.K);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and known to be
   const int wm = wave / C::WN, wn = wave % C::WN;
   float* part = a.part + (int64_t)split * a.M * a.N;
   auto store = [&](float16v (&acc)[C::FM][C::FN]) {
@@ -755,7 +762,7 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
   const int G = gridDim.x, w = blockIdx.x;
   const int n_items = (a.n_ids - w + G - 1) / G;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and known to be
   const int wm = wave / C::WN, wn = wave % C::WN;
   float* stage = reinterpret_cast<float*>(smem_raw + C::LDS_BYTES) + wave * DW_STAGE_FLOATS;
 
