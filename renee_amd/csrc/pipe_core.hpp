@@ -67,7 +67,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 // LDS), which makes each wave wait for the stage it has just requested.  The waits for these fetches are
 // the explicit ones in run(); the compiler's own vmcnt bookkeeping for other loads and stores stays
 // correct without knowing about them (operations return in order, so it can only wait longer than
-// needed).  NT marks the fetch non-temporal: for data read once, so that it does not displace reused
+// needed).  M0 is a reserved register (the compiler only ever loads it right in front of an instruction
+// that reads it), so writing it inside the asm block needs no clobber.  NT marks the fetch non-temporal: for data read once, so that it does not displace reused
 // lines from the L2.
 __device__ __forceinline__ uint32_t lds_addr(void* p) { return (uint32_t)(uintptr_t)(XFC_LDS void*)p; }
 // address = uniform 64-bit base + per-lane 32-bit offset
