@@ -70,6 +70,12 @@ __device__ __forceinline__ void wait_vmcnt() {
 // needed).  M0 is a reserved register (the compiler only ever loads it right in front of an instruction
 // that reads it), so writing it inside the asm block needs no clobber.  NT marks the fetch non-temporal: for data read once, so that it does not displace reused
 // lines from the L2.
+// Marks a value the caller knows to be wave-uniform as such (scalar registers, scalar arithmetic).
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uint64_t)v);
+  return (int64_t)(((uint64_t)hi << 32) | (uint64_t)lo);
+}
 __device__ __forceinline__ uint32_t lds_addr(void* p) { return (uint32_t)(uintptr_t)(XFC_LDS void*)p; }
 // address = uniform 64-bit base + per-lane 32-bit offset
 template <bool NT = false>
@@ -156,12 +162,12 @@ struct PipeCore {
     int kmax, kin;       // limit of k; per-thread k offset inside the stage (KC: chunk*8, MC: k-row in group)
     int kgrp[CH];        // uniform: first k-row of each instruction (MC), 0 (KC)
     __device__ __forceinline__ void init(const Operand& o, int k_begin, int wave, int lane) {
-      base = reinterpret_cast<const char*>(o.p);
+      base = reinterpret_cast<const char*>(uniform64(reinterpret_cast<int64_t>(o.p)));
       kmax = o.kmax;
       const int sub = lane / CPI, pc = lane % CPI;
       if constexpr (KC) {
         kstep = (int64_t)BK * 2;
-        kbytes = (int64_t)k_begin * 2;
+        kbytes = uniform64((int64_t)k_begin * 2);
         const int c = pc ^ kc_swz<BK>(wave * RPI + sub);  // the swizzle does not depend on i (NW is even)
         kin = c * 8;
 #pragma unroll
@@ -169,20 +175,20 @@ struct PipeCore {
           const int row0 = o.r0 + (i * NW + wave) * RPI;
           const int g = row0 < o.rmax ? row0 : o.rmax - 1;
           const int row = row0 + sub < o.rmax ? row0 + sub : o.rmax - 1;
-          grp[i] = (int64_t)g * o.ld * 2;
+          grp[i] = uniform64((int64_t)g * o.ld * 2);
           voff[i] = (uint32_t)(row - g) * (uint32_t)(o.ld * 2) + (uint32_t)c * 16u;
           kgrp[i] = 0;
         }
       } else {
-        kstep = (int64_t)BK * o.ld * 2;
-        kbytes = (int64_t)k_begin * o.ld * 2;
+        kstep = uniform64((int64_t)BK * o.ld * 2);
+        kbytes = uniform64((int64_t)k_begin * o.ld * 2);
         const int c = pc ^ mc_swz(wave * RPI + sub);
         const int col = o.r0 + c * 8 < o.rmax ? o.r0 + c * 8 : o.rmax - 8;
         kin = sub;
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
           kgrp[i] = (i * NW + wave) * RPI;
-          grp[i] = (int64_t)kgrp[i] * o.ld * 2;
+          grp[i] = uniform64((int64_t)kgrp[i] * o.ld * 2);
           voff[i] = (uint32_t)sub * (uint32_t)(o.ld * 2) + (uint32_t)col * 2u;
         }
       }
