@@ -1,13 +1,22 @@
 #!/usr/bin/env python3
 """XFC step benchmark on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu] [--no-others]
 
 A "step" is one pass of the hot path over one synthetic batch: fwd + loss
 gradient (G), dX, dW fused with the SGD-momentum update of the fp16 label
 matrix.  Inputs are resident in HBM before the timed region starts.  Prints ONE
 JSON line.  The workload is BASELINE.json's headline configuration (configs[2]:
 batch 512, d = 768, L = 1,310,720, fp16 storage, fp32 accumulate).
+
+Every timed step starts from the stated data: W ~ N(0, 0.02) as initialised and
+the momentum left by the first step.  W and M are put back (xfc_copy) before each
+timed step, outside the step's event pair, because at lr = 0.05 on these inputs
+W moves by O(100 %) per step and MFMA throughput depends on the operand values.
+`ms_per_step` is the mean of the K per-step HIP event intervals; the same K steps
+run back to back without the restore are reported once as `drifting_ms_per_step`.
+The other BASELINE configurations (1, 3 with its top-5 / top-100 scorers, 4) are
+timed the same way with fewer steps and reported under `other_configs`.
 """
 from __future__ import annotations
 
@@ -23,9 +32,32 @@ sys.path.insert(0, ROOT)
 MFMA_F16_PEAK_TFLOPS = 2516.6   # MI355X dense fp16, AMD's published figure
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
-# HBM bytes per launch of the dW+update kernel at configs[2]: rocprofv3 --pmc FETCH_SIZE (2,860,723.5 KiB,
-# x2.000 from the 1 GiB copy) + WRITE_SIZE (3,932,160 KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
+# HBM bytes per launch of the dW+update kernel: rocprofv3 --pmc FETCH_SIZE (KiB, x2.000 from the 1 GiB
+# copy in the same run) + WRITE_SIZE (KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
 DW_UPDATE_TRAFFIC_BYTES = {2: (2 * 2820425.4 + 3932160.0) * 1024.0}
+
+
+def _oracle_steps(B, L, d, c, seed, n_max, budget_s, warm):
+    import torch
+
+    from oracle import xfc_oracle as O
+    from renee_amd import synth
+
+    X = synth.make_X(B, d, seed)
+    W = synth.make_W(L, d, seed)
+    M = torch.zeros_like(W)
+    P = synth.make_positives(B, L, c["kmax"], c["kmean"], c["zipf"], seed)
+    px, py = P.coo()
+    times = []
+    t_all = time.perf_counter()
+    for i in range(n_max):
+        t0 = time.perf_counter()
+        r = O.step(X, W, M, px, py, 0.05, 0.9, 0.0, 1.0)
+        W, M = r["W"], r["M"]
+        times.append(time.perf_counter() - t0)
+        if i >= warm + 4 and time.perf_counter() - t_all > budget_s:
+            break
+    return sorted(times[warm:])
 
 
 def cpu_baseline(cfg: int, d: int, seed: int):
@@ -33,7 +65,6 @@ def cpu_baseline(cfg: int, d: int, seed: int):
     host's cores on a label slice of the same workload, scaled to the full label count."""
     import torch
 
-    from oracle import xfc_oracle as O
     from renee_amd import synth
 
     c = synth.CONFIGS[cfg]
@@ -41,60 +72,49 @@ def cpu_baseline(cfg: int, d: int, seed: int):
     Ls = min(L, 131072)
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
     torch.set_num_threads(threads)
-    X = synth.make_X(B, d, seed)
-    W = synth.make_W(Ls, d, seed)
-    M = torch.zeros_like(W)
-    P = synth.make_positives(B, Ls, c["kmax"], c["kmean"], c["zipf"], seed)
-    px, py = P.coo()
-    times = []
-    t_all = time.perf_counter()
-    for i in range(8):
-        t0 = time.perf_counter()
-        r = O.step(X, W, M, px, py, 0.05, 0.9, 0.0, 1.0)
-        W, M = r["W"], r["M"]
-        times.append(time.perf_counter() - t0)
-        if i >= 2 and time.perf_counter() - t_all > 25.0:
-            break
-    t = sorted(times[1:])[len(times[1:]) // 2]  # median, first step dropped
+    ts = _oracle_steps(B, Ls, d, c, seed, 8, 20.0, 1)
+    t = ts[len(ts) // 2]
     t_full = t * (L / Ls)
     return {"value": B / t_full, "unit": "samples/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"B={B}, d={d}, label slice {Ls} of {L} (fp32 torch CPU ops, median of {len(times) - 1} steps "
+            "sample": f"B={B}, d={d}, label slice {Ls} of {L} (fp32 torch CPU ops, median of {len(ts)} steps "
                       f"= {t:.3f} s, scaled x{L / Ls:.0f} to the full label count)",
             "gflops": 6.0 * B * Ls * d / t / 1e9}
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (1..4)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--calibrate", action="store_true",
-                    help="after the timed region, run one 1 GiB xfc_copy (the known-size kernel the traffic "
-                         "counters are scaled by when this command runs under rocprofv3 --pmc)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (label sharding across GPUs is design-only); use --gpus 1",
-              file=sys.stderr)
-        return 2
+def cpu_baseline_cfg0(d: int, seed: int):
+    """BASELINE configs[0] as it stands: batch 32, L = 131,072, fp32, the whole step on the host's
+    cores, 2 warm-up steps, median and minimum of at least 5 timed steps, nothing scaled."""
+    import torch
 
+    from renee_amd import synth
+
+    c = synth.CONFIGS[0]
+    B, L = c["B"], c["L"]
+    ts = _oracle_steps(B, L, d, c, seed, 12, 10.0, 2)
+    t = ts[len(ts) // 2]
+    return {"value": B / t, "unit": "samples/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"BASELINE configs[0] unscaled: B={B}, d={d}, L={L}, fp32 torch CPU ops, 2 warm-up steps, "
+                      f"median of {len(ts)} steps = {t:.4f} s (min {ts[0]:.4f} s)",
+            "s_per_step_median": t, "s_per_step_min": ts[0], "gflops": 6.0 * B * L * d / t / 1e9}
+
+
+def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: bool = True, scorers: bool = False):
+    """Times `steps` steps of one BASELINE configuration, each from the same (W0, M1) state."""
     import torch
 
     from renee_amd import XFCLayer, synth
+    from renee_amd._lib import check, lib
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        return 3
-    dev = torch.device("cuda:0")
-    c = synth.CONFIGS[args.config]
+    c = synth.CONFIGS[cfg]
     B, L, d = c["B"], c["L"], synth.D_MODEL
-    layer = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=0.0, seed=args.seed)
-    X = synth.make_X(B, d, args.seed, dev).half()
-    P = synth.make_positives(B, L, c["kmax"], c["kmean"], c["zipf"], args.seed)
+    layer = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=0.0, seed=seed)
+    X = synth.make_X(B, d, seed, dev).half()
+    P = synth.make_positives(B, L, c["kmax"], c["kmean"], c["zipf"], seed)
     rowptr = torch.from_numpy(P.rowptr).to(dev)
     colidx = torch.from_numpy(P.colidx).to(dev)
+    h = lib()
+    st = torch.cuda.current_stream().cuda_stream
+    nbytes = L * d * 2
 
     def step(ev=None):
         if ev:
@@ -109,41 +129,133 @@ def main() -> int:
         if ev:
             ev[3].record()
 
-    for _ in range(args.warmup):
+    # the state every timed step starts from: W as initialised, M as the first step leaves it
+    W0 = layer.xfc_weight.clone()
+    step()
+    M1 = layer.momentum_buffer.clone()
+
+    def restore():
+        check(h.xfc_copy(W0.data_ptr(), layer.xfc_weight.data_ptr(), nbytes, st), "xfc_copy")
+        check(h.xfc_copy(M1.data_ptr(), layer.momentum_buffer.data_ptr(), nbytes, st), "xfc_copy")
+
+    for _ in range(warmup):
+        restore()
         step()
     torch.cuda.synchronize()
     # events are recorded on torch's current stream, which is the stream every kernel is launched on
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
+        restore()
         step(evs[i])
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    k_ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / args.steps for i in range(3)]
+    wall_with_restore = time.perf_counter() - t0
+    ms_per_step = sum(e[0].elapsed_time(e[3]) for e in evs) / steps
+    k_ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / steps for i in range(3)]
+    out = {"B": B, "L": L, "d": d, "nnz": P.nnz, "zipf": c["zipf"], "ms_per_step": ms_per_step, "k_ms": k_ms,
+           "wall_s_incl_restore": wall_with_restore}
+    if drifting:
+        restore()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        out["drifting_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+    if scorers:
+        restore()
+        for K in (5, 100):
+            layer.topk(X, K)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n = 3
+            e0.record()
+            for _ in range(n):
+                layer.topk(X, K)
+            e1.record()
+            torch.cuda.synchronize()
+            out[f"top{K}_ms"] = e0.elapsed_time(e1) / n
+    del layer, W0, M1
+    torch.cuda.empty_cache()
+    return out
+
+
+def summarise(r):
+    """Per-configuration figures from time_config's result."""
+    B, L, d = r["B"], r["L"], r["d"]
     gemm_flop = 2.0 * B * L * d
-    step_tflops = 3 * gemm_flop / (ms_per_step * 1e-3) / 1e12
+    ms = r["ms_per_step"]
+    tf = 3 * gemm_flop / (ms * 1e-3) / 1e12
+    s = {"workload": f"batch {B}, d={d}, L={L}, {r['nnz']} positives (Zipf s={r['zipf']})",
+         "ms_per_step": ms, "samples_per_s": B / (ms * 1e-3), "step_tflops": tf,
+         "mfma_peak_frac": tf / MFMA_F16_PEAK_TFLOPS,
+         "kernels_ms": {"fwd_grad(+bucket)": r["k_ms"][0], "dx(+reduce)": r["k_ms"][1], "dw_update": r["k_ms"][2]},
+         "w_update_gbs": 8.0 * L * d / (r["k_ms"][2] * 1e-3) / 1e9,
+         "w_update_hbm_frac": 8.0 * L * d / (r["k_ms"][2] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    for k in ("drifting_ms_per_step", "top5_ms", "top100_ms"):
+        if k in r:
+            s[k] = r[k]
+    if "top5_ms" in r:
+        s["top5_tflops"] = gemm_flop / (r["top5_ms"] * 1e-3) / 1e12
+    return s
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (1..4)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-others", action="store_true", help="skip the other BASELINE configurations")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="after the timed region, run one 1 GiB xfc_copy (the known-size kernel the traffic "
+                         "counters are scaled by when this command runs under rocprofv3 --pmc)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (label sharding across GPUs is design-only); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    dev = torch.device("cuda:0")
+    r = time_config(args.config, args.steps, args.warmup, args.seed, dev)
+    s = summarise(r)
+    B, L, d = r["B"], r["L"], r["d"]
+    gemm_flop = 2.0 * B * L * d
+    k_ms = r["k_ms"]
     upd_bytes = 8.0 * L * d  # read W, read M, write W, write M in fp16
     achieved = upd_bytes / (k_ms[2] * 1e-3) / 1e9
+    traffic = DW_UPDATE_TRAFFIC_BYTES.get(args.config)
     out = {
         "metric": "XFC fwd+bwd+update samples/sec at d=768,L=1.31M fp16; % MFMA fp16 peak",
-        "value": B / (ms_per_step * 1e-3),
+        "value": s["samples_per_s"],
         "unit": "samples/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": s["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"BASELINE configs[{args.config}]: XFC step, batch {B}, d={d}, L={L}, fp16 W/M/G, "
-                               f"fp32 accumulate, {P.nnz} positives (Zipf s={c['zipf']})",
-                   "batch": B, "d": d, "labels": L, "lr": 0.05, "momentum": 0.9},
-        "step_tflops": step_tflops,
-        "mfma_peak_frac": step_tflops / MFMA_F16_PEAK_TFLOPS,
-        "kernels_ms": {"fwd_grad(+bucket)": k_ms[0], "dx(+reduce)": k_ms[1], "dw_update": k_ms[2]},
+                               f"fp32 accumulate, {r['nnz']} positives (Zipf s={r['zipf']})",
+                   "batch": B, "d": d, "labels": L, "lr": 0.05, "momentum": 0.9,
+                   "timed_state": "every timed step starts from W ~ N(0,0.02) as initialised and the momentum of "
+                                  "step 1 (restored before each step, outside the timed interval)"},
+        "timing": "mean of per-step HIP event intervals on the launch stream",
+        "drifting_ms_per_step": s.get("drifting_ms_per_step"),
+        "step_tflops": s["step_tflops"],
+        "mfma_peak_frac": s["mfma_peak_frac"],
+        "kernels_ms": s["kernels_ms"],
         "kernels_tflops": {"fwd_grad": gemm_flop / k_ms[0] / 1e9, "dx": gemm_flop / k_ms[1] / 1e9,
                            "dw_update": gemm_flop / k_ms[2] / 1e9},
         "roofline": {"kernel": "dw_kernel<DW_UPDATE> (dW GEMM + SGD-momentum update)", "bound": "hbm",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": DW_UPDATE_TRAFFIC_BYTES.get(args.config)},
+                     "traffic": traffic,
+                     "achieved_incl_measured_traffic": None if traffic is None else traffic / (k_ms[2] * 1e-3) / 1e9},
     }
     if args.calibrate:
         from renee_amd._lib import check, lib
@@ -154,8 +266,19 @@ def main() -> int:
         check(lib().xfc_copy(src.data_ptr(), dst.data_ptr(), src.numel() * 2,
                              torch.cuda.current_stream().cuda_stream), "xfc_copy")
         torch.cuda.synchronize()
+        del src, dst
+    if not args.no_others:
+        others = {}
+        for cfg, n in ((1, 20), (3, 6), (4, 3)):
+            if cfg == args.config:
+                continue
+            others[f"configs[{cfg}]"] = summarise(time_config(cfg, n, 2, args.seed, dev, drifting=False,
+                                                              scorers=(cfg == 3)))
+            others[f"configs[{cfg}]"]["steps"] = n
+        out["other_configs"] = others
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.config, d, args.seed)
+        out["cpu_baseline_cfg0"] = cpu_baseline_cfg0(d, args.seed)
     print(json.dumps(out))
     return 0
 

@@ -173,6 +173,8 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* M, int6
  *     fp16 values.  xfc_topk_workspace_bytes() asks for all B rows at once (B*round_up(L,8)*2
  *     bytes); any 16-byte aligned workspace that holds min(B, 256) rows is accepted and the
  *     rows are then processed in blocks of a multiple of 256.
+ * Scores are expected to be finite: NaN and -inf are never selected by the K <= 8 pass, and a row with
+ * fewer than K selectable scores reports (-inf, numy-1) in the remaining places.
  * Workspace: xfc_topk_workspace_bytes(B, L, K) bytes.
  */
 size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K);

@@ -13,12 +13,33 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the global->LDS fetches list M0 as clobbered on purpose; hipcc notes that the register is reserved
+    "-Wno-inline-asm",
 ]
+# The kernels schedule their own waits around inline-asm fetches (csrc/pipe_core.hpp); they were validated
+# on the GPU with this compiler.  Another version may schedule around the asm differently: rerun the GPU
+# tests before trusting a build made with it.
+VALIDATED_HIPCC = "7.2.26015"
+
+
+def hipcc_version(hipcc: str) -> str:
+    try:
+        out = subprocess.run([hipcc, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True).stdout
+    except OSError:
+        return "unknown"
+    for line in out.splitlines():
+        if line.startswith("HIP version:"):
+            return line.split(":", 1)[1].strip()
+    return "unknown"
 
 
 def build(verbose: bool = False) -> str:
     """Compile the library in-tree and return its path."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    ver = hipcc_version(hipcc)
+    if not ver.startswith(VALIDATED_HIPCC):
+        print(f"renee_amd.build: warning: hipcc {ver} is not the validated {VALIDATED_HIPCC}; "
+              "run the GPU test suite before using this build", file=sys.stderr, flush=True)
     cmd = [hipcc, *HIPCC_FLAGS, *SOURCES, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)

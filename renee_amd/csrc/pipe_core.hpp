@@ -67,9 +67,12 @@ __device__ __forceinline__ void wait_vmcnt() {
 // LDS), which makes each wave wait for the stage it has just requested.  The waits for these fetches are
 // the explicit ones in run(); the compiler's own vmcnt bookkeeping for other loads and stores stays
 // correct without knowing about them (operations return in order, so it can only wait longer than
-// needed).  M0 is a reserved register (the compiler only ever loads it right in front of an instruction
-// that reads it), so writing it inside the asm block needs no clobber.  NT marks the fetch non-temporal: for data read once, so that it does not displace reused
-// lines from the L2.
+// needed).  M0 is a reserved register: the compiler never keeps a value of its own there, it only loads
+// it in front of an instruction that reads it.  The asm statements still list it as clobbered, so that the
+// pass which hoists and merges M0 initialisations sees a definition here and never moves one of the
+// compiler's own M0 loads across a fetch (hipcc warns that the register is reserved; the build silences
+// that one warning).  NT marks the fetch non-temporal: for data read once, so that it does not displace
+// reused lines from the L2.
 // Marks a value the caller knows to be wave-uniform as such (scalar registers, scalar arithmetic).
 __device__ __forceinline__ int64_t uniform64(int64_t v) {
   const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
@@ -88,18 +91,18 @@ __device__ __forceinline__ void load16_to_lds(const void* ubase, uint32_t voff, 
   const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b0);
   const uint64_t b = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
   if constexpr (NT)
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m), "v"(voff), "s"(b) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m), "v"(voff), "s"(b) : "memory", "m0");
   else
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(voff), "s"(b) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(voff), "s"(b) : "memory", "m0");
 }
 // address = per-lane 64-bit pointer
 template <bool NT = false>
 __device__ __forceinline__ void load16_to_lds(const void* g, void* lds_base) {
   const uint32_t m = lds_addr(lds_base);
   if constexpr (NT)
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(m), "v"(g) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(m), "v"(g) : "memory", "m0");
   else
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m), "v"(g) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m), "v"(g) : "memory", "m0");
 }
 
 template <int BK>

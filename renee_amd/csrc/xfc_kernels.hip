@@ -952,11 +952,16 @@ hipError_t raise_lds_limit(int lds) {
   return e;
 }
 
+// Launches Kernel and returns XFC_OK or XFC_ERR_HIP; nothing is launched when the LDS limit cannot be raised.
 template <auto Kernel, class A>
-void launch_k(dim3 g, dim3 b, int lds, hipStream_t st, const A& args) {
-  // a failure stays recorded as the runtime's last error, which check_launch() reports
-  if (raise_lds_limit<Kernel>(lds) != hipSuccess) return;
+int launch_k(dim3 g, dim3 b, int lds, hipStream_t st, const A& args) {
+  const hipError_t e = raise_lds_limit<Kernel>(lds);
+  if (e != hipSuccess) {
+    fprintf(stderr, "xfc: cannot raise the dynamic LDS limit to %d bytes: %s\n", lds, hipGetErrorString(e));
+    return XFC_ERR_HIP;
+  }
   hipLaunchKernelGGL(Kernel, g, b, lds, st, args);
+  return check_launch();
 }
 
 int num_cus() {
@@ -1016,18 +1021,16 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   if (grid > ids) grid = ids;                    // ids is a multiple of 8
   dim3 g((unsigned)grid), b(FwdCore::NT);
   if (mode == FWD_GRAD && loss_part) {
-    launch_k<fwd_kernel<FWD_GRAD, false, true>>(g, b, FWD_LDS_BYTES, st, a);
-    int rc = check_launch();
+    int rc = launch_k<fwd_kernel<FWD_GRAD, false, true>>(g, b, FWD_LDS_BYTES, st, a);
     if (rc) return rc;
     hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(64), 0, st, loss_part, (int)grid, loss_out);
     return check_launch();
   }
-  if (mode == FWD_GRAD) launch_k<fwd_kernel<FWD_GRAD, false>>(g, b, FWD_LDS_BYTES, st, a);
-  else if (mode == FWD_SIGMOID && beta != 0.f) launch_k<fwd_kernel<FWD_SIGMOID, true>>(g, b, FWD_LDS_BYTES, st, a);
-  else if (mode == FWD_SIGMOID && alpha == 1.0f) launch_k<fwd_kernel<FWD_SIGMOID_PLAIN, false>>(g, b, FWD_LDS_BYTES, st, a);
-  else if (mode == FWD_SIGMOID) launch_k<fwd_kernel<FWD_SIGMOID, false>>(g, b, FWD_LDS_BYTES, st, a);
-  else launch_k<fwd_kernel<FWD_LINEAR, false>>(g, b, FWD_LDS_BYTES, st, a);
-  return check_launch();
+  if (mode == FWD_GRAD) return launch_k<fwd_kernel<FWD_GRAD, false>>(g, b, FWD_LDS_BYTES, st, a);
+  if (mode == FWD_SIGMOID && beta != 0.f) return launch_k<fwd_kernel<FWD_SIGMOID, true>>(g, b, FWD_LDS_BYTES, st, a);
+  if (mode == FWD_SIGMOID && alpha == 1.0f) return launch_k<fwd_kernel<FWD_SIGMOID_PLAIN, false>>(g, b, FWD_LDS_BYTES, st, a);
+  if (mode == FWD_SIGMOID) return launch_k<fwd_kernel<FWD_SIGMOID, false>>(g, b, FWD_LDS_BYTES, st, a);
+  return launch_k<fwd_kernel<FWD_LINEAR, false>>(g, b, FWD_LDS_BYTES, st, a);
 }
 
 // Split count for dX: a multiple of 8 slices of the label axis (workgroup ids are dealt round-robin over
@@ -1063,8 +1066,7 @@ int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float*
   a.M = M; a.N = N; a.K = K;
   const int64_t grid = (int64_t)a.tiles_m * a.tiles_n * a.splits;
   if (grid <= 0 || M <= 0 || N <= 0) return XFC_OK;
-  launch_k<dx_kernel>(dim3((unsigned)grid), dim3(DxCore::NT), DX_LDS_BYTES, st, a);
-  int rc = check_launch();
+  int rc = launch_k<dx_kernel>(dim3((unsigned)grid), dim3(DxCore::NT), DX_LDS_BYTES, st, a);
   if (rc) return rc;
   const int64_t nq = (int64_t)M * (N / 4);
   hipLaunchKernelGGL(dx_reduce_kernel, dim3((unsigned)ceil_div(nq, 256)), dim3(256), 0, st, a.part, out, ldo, M, N,
@@ -1081,9 +1083,8 @@ int launch_dw(int mode, DwArgs a, hipStream_t st) {
   a.n_ids = (int)ids;
   int64_t grid = 2 * (int64_t)round_up(num_cus(), 8);  // two resident workgroups per CU
   if (grid > ids) grid = ids / 8 * 8 > 0 ? ids / 8 * 8 : ids;
-  if (mode == DW_UPDATE) launch_k<dw_kernel<DW_UPDATE>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
-  else launch_k<dw_kernel<DW_OUT>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
-  return check_launch();
+  if (mode == DW_UPDATE) return launch_k<dw_kernel<DW_UPDATE>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  return launch_k<dw_kernel<DW_OUT>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
 }
 
 int launch_generic(const void* in1, int64_t as0, int64_t as1, const void* in2, int64_t bs0, int64_t bs1, void* out,
@@ -1280,7 +1281,7 @@ int xfc_dw_update(const void* G, int64_t ldg, const void* X, int64_t ldx, void* 
                   int64_t B, int64_t L, int64_t d, float lr, float momentum, float weight_decay, float* dW_out,
                   int64_t ld_dw, void* stream) {
   if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
-  if (L == 0 || d == 0) return XFC_OK;
+  if (L == 0 || d == 0 || B == 0) return XFC_OK;  // an empty batch is not a step: W and M stay as they are
   if (!G || !X || !W || !Mo) return XFC_ERR_INVALID;
   if (ldg % 8 || ldx % 8 || ldw % 8 || ldm % 8 || d % 8 || !aligned16(G) || !aligned16(X) || !aligned16(W) ||
       !aligned16(Mo))
@@ -1299,6 +1300,8 @@ int xfc_dw(const void* G, int64_t ldg, const void* X, int64_t ldx, float* grad, 
            int64_t d, float beta, void* stream) {
   if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
   if (L == 0 || d == 0) return XFC_OK;
+  if (B == 0 && beta == 1.0f) return XFC_OK;  // an empty micro-batch adds nothing
+  if (B == 0) return XFC_ERR_INVALID;          // beta != 1 with no rows would only rescale grad: not a dW call
   if (!G || !X || !grad) return XFC_ERR_INVALID;
   if (ldg % 8 || ldx % 8 || d % 8 || ld_grad % 4 || !aligned16(G) || !aligned16(X) || !aligned16(grad))
     return XFC_ERR_ALIGN;
@@ -1398,8 +1401,7 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   a.cand_v = reinterpret_cast<float*>(workspace);
   a.cand_i = reinterpret_cast<int32_t*>(a.cand_v + (size_t)a.n_groups * B * K);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  launch_k<topk_kernel>(dim3((unsigned)grid), dim3(TopkCore::NT), TOPK_LDS_BYTES, st, a);
-  int rc = check_launch();
+  int rc = launch_k<topk_kernel>(dim3((unsigned)grid), dim3(TopkCore::NT), TOPK_LDS_BYTES, st, a);
   if (rc) return rc;
   hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)B), dim3(64), 0, st, a.cand_v, a.cand_i, (int)B, a.n_groups, K,
                      numy, values, indices);

@@ -27,13 +27,16 @@ def _round_up(a: int, b: int) -> int:
 
 
 class _Workspace:
-    """One growable byte buffer per device, handed to calls that need scratch."""
+    """Scratch for the bare six-argument xfc_gemm: one growable byte buffer per (device, stream), so
+    calls on different streams never share one.  XFCLayer does not use it: a layer owns a workspace of
+    fixed size, allocated when the layer is built (the reference preallocates its large buffers for the
+    same reason, dl_base.py:175-187)."""
 
     def __init__(self):
         self._buf = {}
 
-    def get(self, device: torch.device, nbytes: int) -> torch.Tensor:
-        key = (device.type, device.index)
+    def get(self, device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+        key = (device.type, device.index, int(stream))
         buf = self._buf.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
@@ -47,6 +50,14 @@ _workspace = _Workspace()
 def _require(cond: bool, msg: str, exc=RuntimeError):
     if not cond:
         raise exc(msg)
+
+
+def gemm_workspace_bytes(in1_strides, in2_strides, M: int, N: int, K: int, apply_sigmoid: bool) -> int:
+    """Scratch the six-argument call needs: only the row x row mode (contraction over the long axis,
+    split; xfc_gemm_kernel.cu:151) uses any.  The column x row mode (dW: M = labels, N = dims) must not
+    be sized by the split plan, which would ask for splits * M * N * 4 bytes (tens of gigabytes)."""
+    row_row = (not apply_sigmoid) and in1_strides[1] == 1 and in2_strides[1] == 1 and in1_strides[0] != 1
+    return int(lib().xfc_gemm_workspace_bytes(M, N, K)) if row_row else 0
 
 
 def xfc_gemm(mat_in1: torch.Tensor, mat_in2: torch.Tensor, mat_out: torch.Tensor,
@@ -66,9 +77,9 @@ def xfc_gemm(mat_in1: torch.Tensor, mat_in2: torch.Tensor, mat_out: torch.Tensor
     M, N = mat_out.shape
     K = mat_in2.shape[0]
     L = lib()
-    ws_bytes = L.xfc_gemm_workspace_bytes(M, N, K) if not apply_sigmoid else 0
+    ws_bytes = gemm_workspace_bytes(mat_in1.stride(), mat_in2.stride(), M, N, K, apply_sigmoid)
     with torch.cuda.device(mat_out.device):
-        ws = _workspace.get(mat_out.device, ws_bytes)
+        ws = _workspace.get(mat_out.device, _stream(mat_out), ws_bytes)
         rc = L.xfc_gemm(mat_in1.data_ptr(), mat_in1.shape[0], mat_in1.shape[1], mat_in1.stride(0), mat_in1.stride(1),
                         mat_in2.data_ptr(), mat_in2.shape[0], mat_in2.shape[1], mat_in2.stride(0), mat_in2.stride(1),
                         mat_out.data_ptr(), M, N, mat_out.stride(0), mat_out.stride(1),
@@ -107,10 +118,11 @@ def read_sparse_labels(path: str):
     return rowptr, np.asarray(colidx, dtype=np.int32), (rows, cols)
 
 
-def batch_positives(rowptr, colidx, ids, start_label: int = 0, end_label: int | None = None):
+def batch_positives(rowptr, colidx, ids, start_label: int = 0, end_label: int | None = None, device=None):
     """The collator's label tensor for a batch (dl_base.py:934-936: labels[full_ids].tocoo() as a
     2 x nnz LongTensor, rows ascending), optionally restricted and re-based to one rank's label columns
-    (main.py:94-97)."""
+    (main.py:94-97).  The result is a CPU tensor, as the collator's is, unless `device` is given;
+    XFCLayer moves index tensors to its GPU itself."""
     import numpy as np
 
     rows, cols = [], []
@@ -122,7 +134,8 @@ def batch_positives(rowptr, colidx, ids, start_label: int = 0, end_label: int | 
             c = c[c >= start_label]
         rows.append(np.full(c.shape[0], b, dtype=np.int64))
         cols.append(c.astype(np.int64) - start_label)
-    return torch.from_numpy(np.stack([np.concatenate(rows), np.concatenate(cols)])) if rows else torch.zeros(2, 0, dtype=torch.int64)
+    z = torch.from_numpy(np.stack([np.concatenate(rows), np.concatenate(cols)])) if rows else torch.zeros(2, 0, dtype=torch.int64)
+    return z if device is None else z.to(device)
 
 
 def coo_to_csr(pos_x: torch.Tensor, pos_y: torch.Tensor, num_rows: int):
@@ -141,15 +154,23 @@ class XFCLayer:
     any label count is accepted.  W and the momentum are fp16 and stay
     resident; G (`outsoft`, dl_base.py:176) is preallocated for max_batch rows
     with its rows padded to a multiple of 8 labels.
+
+    Every buffer, the kernels' workspace included, is allocated here and never
+    again (dl_base.py:175-187 preallocates for the same reason): a layer's calls
+    can be captured into a HIP graph without a sizing pass, and two layers never
+    share scratch, so they may run on two streams at once.  One layer's calls
+    must stay on one stream at a time.  `max_positives` bounds the label pairs
+    of one batch (default 64 per row of max_batch).
     """
 
     def __init__(self, numy: int, dims: int, max_batch: int, device="cuda:0", lr: float = 0.05,
                  momentum: float = 0.9, weight_decay: float = 0.0, weight: torch.Tensor | None = None,
-                 seed: int = 0):
+                 seed: int = 0, max_positives: int | None = None):
         self.device = torch.device(device)
         _require(self.device.type == "cuda", "XFCLayer needs a GPU device")
         _require(dims % 8 == 0, "dims must be a multiple of 8")
         self.numy, self.dims, self.max_batch = int(numy), int(dims), int(max_batch)
+        self.max_positives = int(max_positives) if max_positives is not None else 64 * self.max_batch
         self.lr, self.momentum, self.weight_decay = float(lr), float(momentum), float(weight_decay)
         self.ldg = _round_up(self.numy, 8)
         if weight is None:
@@ -168,8 +189,12 @@ class XFCLayer:
         self.outsoft = torch.empty(self.max_batch, self.ldg, device=self.device, dtype=torch.float16)
         self.grad_input = torch.empty(self.max_batch, self.dims, device=self.device, dtype=torch.float32)
         self.xfc_weight_grad = None  # fp32 accumulator, only under split accumulation
+        L = lib()
         with torch.cuda.device(self.device):
-            check(lib().xfc_init(), "xfc_init")
+            check(L.xfc_init(), "xfc_init")
+            need = max(L.xfc_step_workspace_bytes(self.max_batch, self.numy, self.dims, self.max_positives),
+                       L.xfc_topk_workspace_bytes(self.max_batch, self.numy, min(8, self.numy)), 256)
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
 
     # -- helpers ---------------------------------------------------------------------------
     def _x16(self, embed: torch.Tensor) -> torch.Tensor:
@@ -181,6 +206,21 @@ class XFCLayer:
         _require(bsz <= self.max_batch, "batch larger than max_batch")
         return self.outsoft[0:bsz]
 
+    def _index(self, t: torch.Tensor, dtype: torch.dtype, what: str) -> torch.Tensor:
+        """An index tensor as the kernels read it: 1-D, contiguous, of `dtype`, on this layer's GPU.
+        The dtype is checked, never converted (a silent int64 -> int32 pass would hide a caller's
+        mistake); a tensor on another device (the collator's 'z' lives on the CPU) is copied over."""
+        _require(isinstance(t, torch.Tensor) and t.dim() == 1, f"{what} must be a 1-D tensor")
+        _require(t.dtype == dtype, f"{what} must be {dtype}", TypeError)
+        if t.device != self.device:
+            t = t.to(self.device)
+        return t.contiguous()
+
+    def _check_nnz(self, nnz: int) -> None:
+        _require(nnz <= self.max_positives,
+                 f"{nnz} label pairs in one batch exceed max_positives={self.max_positives}; "
+                 "build the layer with a larger max_positives", ValueError)
+
     # -- reference operators ---------------------------------------------------------------
     def xfc_forward(self, embed: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """Logits out = embed . W^T (dl_base.py:568-573)."""
@@ -188,36 +228,33 @@ class XFCLayer:
         bsz = x.shape[0]
         if out is None:
             out = self._g_view(bsz)[:, : self.numy]
-        _require(out.dtype == torch.float16 and out.stride(1) == 1 and tuple(out.shape) == (bsz, self.numy),
-                 "out must be float16 (batch, numy) with unit column stride")
+        _require(out.dtype == torch.float16 and out.stride(1) == 1 and tuple(out.shape) == (bsz, self.numy)
+                 and out.device == self.device,
+                 "out must be float16 (batch, numy) with unit column stride on the layer's device")
         with torch.cuda.device(self.device):
             rc = lib().xfc_logits(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                   out.data_ptr(), out.stride(0), bsz, self.numy, self.dims, _stream(x))
         check(rc, "xfc_logits")
         return out
 
-    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None,
-             max_workspace_bytes: int = 8 << 30):
+    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None):
         """Exact top-K labels per row over all labels (FullPredictor's scoring loop, dl_base.py:736-756,
         with the pad clamp of :782 when numy < the stored label count).  Returns (values fp32, indices
         int64), each (batch, K); ties go to the lower label id.  K <= 128: up to 8 in one fused pass,
-        above that (the final evaluation's K = 100, dl_base.py:817-818) by an exact selection over fp16
-        logits held in the workspace, at most `max_workspace_bytes` of them at a time."""
+        above that (the final evaluation's K = 100, dl_base.py:817-818) by an exact selection over the
+        fp16 logits, which are written to `outsoft` as the reference's scorer does (dl_base.py:745)."""
         x = self._x16(embed)
         bsz = x.shape[0]
         _require(1 <= K <= 128 and K <= self.numy, "K must be in 1..min(128, numy)")
+        _require(bsz <= self.max_batch, "batch larger than max_batch")
         vals = torch.empty(bsz, K, device=self.device, dtype=torch.float32)
         inds = torch.empty(bsz, K, device=self.device, dtype=torch.int64)
         L = lib()
+        ws = self.outsoft if K > 8 else self._ws
         with torch.cuda.device(self.device):
-            need = L.xfc_topk_workspace_bytes(bsz, self.numy, K)
-            if K > 8 and need > max_workspace_bytes:  # rows in blocks of a multiple of 256
-                row_bytes = self.ldg * 2
-                need = max(256, max_workspace_bytes // row_bytes // 256 * 256) * row_bytes
-            ws = _workspace.get(self.device, need)
             rc = L.xfc_topk(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims, bsz, self.numy,
                             self.dims, self.numy if numy is None else int(numy), int(K), vals.data_ptr(),
-                            inds.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))
+                            inds.data_ptr(), ws.data_ptr(), ws.numel() * ws.element_size(), _stream(x))
         check(rc, "xfc_topk")
         return vals, inds
 
@@ -235,20 +272,26 @@ class XFCLayer:
         G = self._g_view(bsz)
         L = lib()
         csr = rowptr is not None
-        nnz = int(colidx.numel() if csr else (0 if pos_x is None else pos_x.numel()))
+        ws = self._ws
+        # every index tensor is validated and brought to this GPU before anything is launched
+        if csr:
+            rowptr = self._index(rowptr, torch.int32, "rowptr")
+            colidx = self._index(colidx, torch.int32, "colidx")
+            _require(rowptr.numel() == bsz + 1, "rowptr must have batch+1 entries")
+            nnz = int(colidx.numel())
+        else:
+            nnz = 0 if pos_x is None else int(pos_x.numel())
+            if nnz:
+                pos_x = self._index(pos_x, torch.int64, "pos_x")
+                pos_y = self._index(pos_y, torch.int64, "pos_y")
+                _require(pos_x.numel() == pos_y.numel(), "pos_x / pos_y length")
+        self._check_nnz(nnz)
         with torch.cuda.device(self.device):
-            ws = _workspace.get(self.device, L.xfc_fwd_grad_workspace_bytes(self.numy, nnz))
             if csr:
-                _require(rowptr.dtype == torch.int32 and colidx.dtype == torch.int32, "CSR must be int32", TypeError)
-                _require(rowptr.numel() == bsz + 1, "rowptr must have batch+1 entries")
                 rc = L.xfc_fwd_grad_csr(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                         rowptr.data_ptr(), colidx.data_ptr(), G.data_ptr(), self.ldg,
                                         bsz, self.numy, self.dims, nnz, lp, ws.data_ptr(), ws.numel(), _stream(x))
             else:
-                if nnz:
-                    _require(pos_x.dtype == torch.int64 and pos_y.dtype == torch.int64, "COO must be int64", TypeError)
-                    _require(pos_x.numel() == pos_y.numel(), "pos_x / pos_y length")
-                    pos_x, pos_y = pos_x.contiguous(), pos_y.contiguous()
                 rc = L.xfc_fwd_grad_coo(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                         pos_x.data_ptr() if nnz else None, pos_y.data_ptr() if nnz else None, nnz,
                                         G.data_ptr(), self.ldg, bsz, self.numy, self.dims, lp,
@@ -261,11 +304,12 @@ class XFCLayer:
         if grad_input is None:
             grad_input = self.grad_input[0:bsz]
         _require(grad_input.dtype == torch.float32 and grad_input.stride(1) == 1 and
-                 tuple(grad_input.shape) == (bsz, self.dims), "grad_input must be float32 (batch, dims)")
+                 tuple(grad_input.shape) == (bsz, self.dims) and grad_input.device == self.device,
+                 "grad_input must be float32 (batch, dims) on the layer's device")
         L = lib()
         G = self._g_view(bsz)
+        ws = self._ws
         with torch.cuda.device(self.device):
-            ws = _workspace.get(self.device, L.xfc_dx_workspace_bytes(bsz, self.numy, self.dims))
             rc = L.xfc_dx(G.data_ptr(), self.ldg, self.xfc_weight.data_ptr(), self.dims, grad_input.data_ptr(),
                           grad_input.stride(0), bsz, self.numy, self.dims, float(scale),
                           ws.data_ptr(), ws.numel(), _stream(G))
@@ -278,8 +322,9 @@ class XFCLayer:
         bsz = x.shape[0]
         G = self._g_view(bsz)
         if dW_out is not None:
-            _require(dW_out.dtype == torch.float32 and dW_out.is_contiguous() and
-                     tuple(dW_out.shape) == (self.numy, self.dims), "dW_out must be contiguous float32 (numy, dims)")
+            _require(dW_out.dtype == torch.float32 and dW_out.is_contiguous() and dW_out.device == self.device and
+                     tuple(dW_out.shape) == (self.numy, self.dims),
+                     "dW_out must be contiguous float32 (numy, dims) on the layer's device")
         with torch.cuda.device(self.device):
             rc = lib().xfc_dw_update(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0),
                                      self.xfc_weight.data_ptr(), self.dims, self.momentum_buffer.data_ptr(), self.dims,
@@ -319,16 +364,26 @@ class XFCLayer:
                 "numy": self.numy, "dims": self.dims, "lr": self.lr, "momentum": self.momentum,
                 "weight_decay": self.weight_decay}
 
-    def load_state_dict(self, state: dict) -> None:
-        """Restore from state_dict(); an fp32 xfc_weight (a reference checkpoint's) is rounded to fp16 once
-        and a missing momentum_buffer starts from zero, as the optimizer's first step does."""
+    def load_state_dict(self, state: dict, optimizer_state: dict | None = None) -> None:
+        """Restore from state_dict().  A reference checkpoint is accepted too: its fp32 `xfc_weight`
+        (dl_base.py:420) is rounded to fp16 once, and `optimizer_state` may be the reference's
+        `xfc_optimizer_state_dict` (dl_base.py:424; torch's optimizer layout, {'state': {0:
+        {'momentum_buffer': fp32 L x d}}, 'param_groups': [...]}), whose momentum buffer is rounded to
+        fp16 the same way.  Without any momentum the buffer starts from zero, as the optimizer's
+        first step does."""
         w = state["xfc_weight"]
         _require(tuple(w.shape) == (self.numy, self.dims), "checkpoint shape does not match this layer")
         self.xfc_weight.copy_(w.to(device=self.device, dtype=torch.float16))
         m = state.get("momentum_buffer")
+        if m is None and optimizer_state is not None:
+            per_param = list(optimizer_state.get("state", {}).values())
+            _require(len(per_param) <= 1, "the XFC optimizer holds one parameter (dl_base.py:222-238)")
+            if per_param:
+                m = per_param[0].get("momentum_buffer")
         if m is None:
             self.momentum_buffer.zero_()
         else:
+            _require(tuple(m.shape) == (self.numy, self.dims), "momentum buffer shape does not match this layer")
             self.momentum_buffer.copy_(m.to(device=self.device, dtype=torch.float16))
         for k in ("lr", "momentum", "weight_decay"):
             if k in state:
@@ -357,9 +412,13 @@ class XFCLayer:
         G = self._g_view(bsz)
         gi = self.grad_input[0:bsz]
         L = lib()
+        rowptr = self._index(rowptr, torch.int32, "rowptr")
+        colidx = self._index(colidx, torch.int32, "colidx")
+        _require(rowptr.numel() == bsz + 1, "rowptr must have batch+1 entries")
         nnz = int(colidx.numel())
+        self._check_nnz(nnz)
+        ws = self._ws
         with torch.cuda.device(self.device):
-            ws = _workspace.get(self.device, L.xfc_step_workspace_bytes(bsz, self.numy, self.dims, nnz))
             rc = L.xfc_step_csr(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                 self.momentum_buffer.data_ptr(), self.dims, rowptr.data_ptr(), colidx.data_ptr(), nnz,
                                 G.data_ptr(), self.ldg, gi.data_ptr(), self.dims, bsz, self.numy, self.dims,

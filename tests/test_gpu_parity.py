@@ -270,8 +270,7 @@ def test_step_under_graph_capture(dev):
     Xd = X.to(dev)
     eager = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=1e-4, weight=W)
     graphed = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=1e-4, weight=W)
-    graphed.step_csr(Xd, rp, ci, scale=2.0)  # warm-up outside capture: sizes the workspace
-    eager.step_csr(Xd, rp, ci, scale=2.0)
+    # no sizing pass for the captured layer: its buffers, workspace included, exist since construction
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
@@ -282,7 +281,7 @@ def test_step_under_graph_capture(dev):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     # the captured call did not run; replay and compare with eager steps, with eager work in between
-    for _ in range(3):
+    for _ in range(4):
         g.replay()
         ge = eager.step_csr(Xd, rp, ci, scale=2.0).clone()
         torch.cuda.synchronize()
@@ -352,3 +351,90 @@ def test_seeded_shape_sweep(dev):
         assert rel(dX[:B], ref["dX"]) <= TOL
         assert rel(lay.xfc_weight, ref["W"]) <= TOL
         assert rel(lay.momentum_buffer, ref["M"]) <= TOL
+
+
+def test_index_tensors_are_checked_and_moved_before_any_launch(dev):
+    """Label tensors arrive from the collator on the CPU (dl_base.py:934-936).  They are copied to the
+    layer's GPU, never dereferenced where they are; a wrong dtype or length raises before a launch."""
+    B, L, d = 64, 3000, 64
+    X, W, P = _problem(B, L, d, seed=21)
+    px, py = P.coo()
+    rp, ci = torch.from_numpy(P.rowptr), torch.from_numpy(P.colidx)
+    lay = XFCLayer(L, d, B, dev, weight=W)
+    Xd = X.to(dev)
+    G_dev = lay.fwd_grad(Xd, px.to(dev), py.to(dev)).clone()
+    G_cpu = lay.fwd_grad(Xd, px, py).clone()                      # CPU COO: moved, same result
+    assert torch.equal(G_dev, G_cpu)
+    G_csr = lay.fwd_grad(Xd, rowptr=rp, colidx=ci).clone()        # CPU CSR
+    assert torch.equal(G_dev, G_csr)
+    marker = lay.outsoft[:B].clone()
+    with pytest.raises(TypeError):
+        lay.fwd_grad(Xd, rowptr=rp.long(), colidx=ci)             # int64 CSR is not silently misread
+    with pytest.raises(TypeError):
+        lay.step_csr(Xd, rp.to(dev), ci.long().to(dev))
+    with pytest.raises(TypeError):
+        lay.fwd_grad(Xd, px.int(), py.int())
+    with pytest.raises(RuntimeError):
+        lay.step_csr(Xd, rp[:-1], ci)                             # rowptr must have B + 1 entries
+    with pytest.raises(RuntimeError):
+        lay.fwd_grad(Xd, px[:-1], py)
+    small = XFCLayer(L, d, B, dev, weight=W, max_positives=4)
+    with pytest.raises(ValueError):
+        small.fwd_grad(Xd, px, py)
+    torch.cuda.synchronize()
+    assert torch.equal(lay.outsoft[:B], marker)                   # nothing ran for the rejected calls
+    gi = lay.step_csr(Xd, rp, ci)                                 # CPU CSR through the one-call step
+    ref = O.step(X.float(), W.float(), torch.zeros(L, d), px, py, 0.05, 0.9, 0.0, 1.0)
+    assert rel(gi, ref["dX"]) <= TOL and rel(lay.xfc_weight, ref["W"]) <= TOL
+
+
+def test_two_layers_on_two_streams(dev):
+    """Each layer owns its scratch, so two layers may run on two streams at once: the results are
+    bit-identical to the same steps run one after the other."""
+    B, L, d = 256, 40000, 256
+    X, W, P = _problem(B, L, d, seed=22)
+    X2, W2, P2 = _problem(B, L, d, seed=23)
+    rp, ci = torch.from_numpy(P.rowptr).to(dev), torch.from_numpy(P.colidx).to(dev)
+    rp2, ci2 = torch.from_numpy(P2.rowptr).to(dev), torch.from_numpy(P2.colidx).to(dev)
+    Xd, X2d = X.to(dev), X2.to(dev)
+
+    def build():
+        return (XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W),
+                XFCLayer(L, d, B, dev, lr=0.02, momentum=0.8, weight=W2))
+
+    sa, sb = build()
+    for _ in range(3):
+        sa.step_csr(Xd, rp, ci, scale=2.0)
+        sb.step_csr(X2d, rp2, ci2, scale=0.5)
+    torch.cuda.synchronize()
+    ca, cb = build()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        with torch.cuda.stream(s1):
+            ca.step_csr(Xd, rp, ci, scale=2.0)
+        with torch.cuda.stream(s2):
+            cb.step_csr(X2d, rp2, ci2, scale=0.5)
+    torch.cuda.synchronize()
+    for serial, conc in ((sa, ca), (sb, cb)):
+        assert torch.equal(serial.xfc_weight, conc.xfc_weight)
+        assert torch.equal(serial.momentum_buffer, conc.momentum_buffer)
+        assert torch.equal(serial.grad_input[:B], conc.grad_input[:B])
+
+
+def test_empty_batch_and_reference_optimizer_state(dev):
+    """B = 0 launches nothing and leaves W and M alone; a reference checkpoint's optimizer state
+    (torch layout, fp32 momentum_buffer) is taken over by load_state_dict."""
+    from renee_amd._lib import lib
+    L, d = 1000, 64
+    W = synth.make_W(L, d, 5).half()
+    lay = XFCLayer(L, d, 8, dev, weight=W)
+    st = torch.cuda.current_stream().cuda_stream
+    rc = lib().xfc_dw_update(lay.outsoft.data_ptr(), lay.ldg, lay.outsoft.data_ptr(), d, lay.xfc_weight.data_ptr(), d,
+                             lay.momentum_buffer.data_ptr(), d, 0, L, d, 0.05, 0.9, 0.0, None, 0, st)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.equal(lay.xfc_weight.cpu(), W) and float(lay.momentum_buffer.abs().max()) == 0.0
+    m32 = torch.randn(L, d) * 0.1
+    lay.load_state_dict({"xfc_weight": W.float()},
+                        optimizer_state={"state": {0: {"momentum_buffer": m32}}, "param_groups": [{"lr": 0.05}]})
+    assert torch.equal(lay.momentum_buffer.cpu(), m32.half())

@@ -96,8 +96,18 @@ def _check_select(dev, X, W, K, numy=None, max_ws=None, vs_oracle=True):
     L = W.shape[0]
     lay = XFCLayer(L, d, B, dev, weight=W)
     print(f"topk-select: B={B} L={L} d={d} K={K} numy={numy} max_ws={max_ws}", flush=True)
-    kw = {} if max_ws is None else {"max_workspace_bytes": max_ws}
-    v, i = lay.topk(X.to(dev), K, numy, **kw)
+    if max_ws is None:
+        v, i = lay.topk(X.to(dev), K, numy)
+    else:
+        # a caller workspace smaller than all rows' logits, straight through the C ABI
+        from renee_amd._lib import check, lib
+        Xd = X.to(dev)
+        ws = torch.empty(max_ws, dtype=torch.uint8, device=dev)
+        v = torch.empty(B, K, device=dev, dtype=torch.float32)
+        i = torch.empty(B, K, device=dev, dtype=torch.int64)
+        check(lib().xfc_topk(Xd.data_ptr(), Xd.stride(0), lay.xfc_weight.data_ptr(), d, B, L, d,
+                             L if numy is None else numy, K, v.data_ptr(), i.data_ptr(), ws.data_ptr(), ws.numel(),
+                             torch.cuda.current_stream().cuda_stream), "xfc_topk")
     v, i = v.cpu(), i.cpu()
     # (a) the selection itself, against a stable sort of the same fp16 logits: exact
     Zg = lay.xfc_forward(X.to(dev)).float().cpu()

@@ -185,3 +185,124 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0, out
     assert "workspace" in out.stdout.lower()
+
+
+def test_gemm_workspace_is_requested_only_for_the_split_mode():
+    """The column x row call the reference makes for dW (out.t(), embed -> L x d, dl_base.py:623) uses
+    no workspace; sizing it by the split plan would ask for tens of gigabytes at the headline shape."""
+    from renee_amd.xfc import gemm_workspace_bytes
+
+    L, B, d = 1310720, 512, 768
+    assert gemm_workspace_bytes((1, L), (d, 1), L, d, B, False) == 0          # dW: G^T view x X
+    assert gemm_workspace_bytes((d, 1), (1, d), B, L, d, True) == 0           # sigmoid: X x W^T view
+    need = gemm_workspace_bytes((L, 1), (d, 1), B, d, L, False)               # dX: G x W, split over labels
+    assert need == lib().xfc_gemm_workspace_bytes(B, d, L) and 0 < need < (1 << 30)
+
+
+def test_empty_batch_is_accepted_without_touching_the_device():
+    h = lib()
+    one = ctypes.c_void_p(16)
+    assert h.xfc_dw_update(one, 8, one, 8, one, 8, one, 8, 0, 8, 8, 0.1, 0.9, 0.0, None, 0, None) == 0
+    assert h.xfc_dw(one, 8, one, 8, one, 8, 0, 8, 8, 1.0, None) == 0
+    assert h.xfc_dw(one, 8, one, 8, one, 8, 0, 8, 8, 0.0, None) == 1
+
+
+# ---------------------------------------------------------------------------------------------------
+# The main loop's hand-counted waits (renee_amd/csrc/pipe_core.hpp, PipeCore::run): a model of what the
+# hardware guarantees, run over the schedule the code issues, for every instantiation in the kernels.
+#   * a wave's global->LDS fetches retire in issue order; other vector-memory operations (an epilogue's
+#     loads and stores) share the counter and may retire at any time relative to the fetches;
+#   * s_waitcnt vmcnt(N) returns once at most N operations are outstanding, whichever they are;
+#   * after the s_barrier that follows it, what one wave knows about its own fetches holds for all.
+# Checked: no stage is read before its fetches are certain to have landed, and no slot is refilled
+# before every wave is past its last read of the stage it held.
+# ---------------------------------------------------------------------------------------------------
+def _pipecore_instantiations():
+    import re
+
+    src = open(os.path.join(ROOT, "renee_amd", "csrc", "xfc_kernels.hip")).read()
+    found = {}
+    for name, args in re.findall(r"using\s+(\w+)\s*=\s*PipeCore<([^>]*)>", src):
+        v = [a.strip() for a in args.split(",")]
+        bm, bn, bk, wm, wn, stages = (int(x) for x in v[:6])
+        loads = (bm * bk // 8 + bn * bk // 8) // (64 * wm * wn)
+        found[name] = (stages, loads)
+    return found
+
+
+def _simulate_ring(stages, loads, item_stages, epilogue_ops, slack=0):
+    """Walks PipeCore::run's schedule for one wave.  Returns a list of error strings (empty = safe)."""
+    errors = []
+    total = sum(item_stages)
+    outstanding = []            # issue-ordered: ('f', stage) per fetch instruction, ('o',) per epilogue op
+    landed = set()              # fetch stages certain to have landed (for every wave, once a barrier passed)
+    released = set()            # stages every wave has finished reading
+    issued = 0
+
+    def issue_one():
+        nonlocal issued
+        s = issued              # stages past the end are the zero-block fetches that keep the count constant
+        prev = s - stages       # the stage that lived in this slot
+        if prev >= 0 and prev < total and prev not in released:
+            errors.append(f"slot of stage {prev} refilled with stage {s} before all waves were past reading it")
+        outstanding.extend([("f", s)] * loads)
+        issued += 1
+
+    def wait_vmcnt_barrier(n):
+        # adversary: epilogue operations retire first, then the oldest fetches, until at most n remain
+        nonlocal outstanding
+        excess = len(outstanding) - n
+        if excess > 0:
+            others = [i for i, op in enumerate(outstanding) if op[0] == "o"][:excess]
+            keep = [op for i, op in enumerate(outstanding) if i not in set(others)]
+            excess -= len(others)
+            outstanding = keep[max(0, excess):]
+        pending = {op[1] for op in outstanding if op[0] == "f"}
+        for s in range(issued):
+            if s not in pending:
+                landed.add(s)
+
+    def read(stage):
+        if stage < total and stage not in landed:
+            errors.append(f"stage {stage} read before its fetches are known to have landed")
+
+    for _ in range(stages - 1):
+        issue_one()
+    wait_vmcnt_barrier((stages - 2) * loads + slack)
+    issue_one()
+    read(0)
+    c = 0
+    drain_all = False
+    for nk in item_stages:
+        for _ in range(nk):
+            read(c)                                  # the sub-steps' fragment reads of stage c
+            wait_vmcnt_barrier(0 if drain_all else (stages - 2) * loads + slack)
+            drain_all = False
+            released.add(c)                          # every wave's reads of stage c precede its barrier arrival
+            issue_one()                              # stage c + STAGES into the slot of stage c
+            read(c + 1)                              # first fragments of the next stage
+            c += 1
+        outstanding.extend([("o",)] * epilogue_ops)  # the epilogue's own loads and stores
+        drain_all = True
+    return errors
+
+
+def test_main_loop_wait_counts_never_expose_a_stage_in_flight():
+    src = open(os.path.join(ROOT, "renee_amd", "csrc", "pipe_core.hpp")).read()
+    # the model below mirrors these statements of PipeCore::run; if they change, so must the model
+    assert src.count("wait_vmcnt_barrier<(STAGES - 2) * LOADS_PER_STAGE>()") == 1
+    assert src.count("wait_lds_vmcnt_barrier<(STAGES - 2) * LOADS_PER_STAGE>()") == 1
+    assert "if (drain_all) { wait_lds_vmcnt_barrier<0>(); drain_all = false; }" in src
+    assert "for (int s = 0; s < STAGES - 1; ++s) issue_one();" in src
+    inst = _pipecore_instantiations()
+    assert {"FwdCore", "DxCore", "DwCore"} <= set(inst)
+    shapes = dict(inst)
+    shapes.update({"three_slots": (3, 8), "four_slots": (4, 4), "five_slots": (5, 2)})  # deeper rings the template allows
+    for name, (stages, loads) in shapes.items():
+        assert stages >= 2 and (stages - 1) * loads < 64, name   # vmcnt is a 6-bit counter
+        for items in ([1], [1, 1, 1], [3, 1, 2], [12], [2] * 7, [16, 16]):
+            for ep in (0, 3, 40):
+                assert _simulate_ring(stages, loads, items, ep) == [], (name, items, ep)
+    # the model does catch a wait that is one stage too permissive
+    for stages, loads in ((3, 8), (4, 4)):
+        assert _simulate_ring(stages, loads, [12], 0, slack=loads) != []
