@@ -32,7 +32,8 @@ enum {
   XFC_ERR_ALIGN = 3,     /* pointer or leading dimension not 16-byte aligned */
   XFC_ERR_WORKSPACE = 4, /* workspace NULL or smaller than *_workspace_bytes() */
   XFC_ERR_HIP = 5,       /* kernel launch failed */
-  XFC_ERR_SHAPE = 6      /* operand shapes disagree / leading dimension too small */
+  XFC_ERR_SHAPE = 6,     /* operand shapes disagree / leading dimension too small */
+  XFC_ERR_LIMIT = 7      /* problem larger than the fixed capacity of a *_static entry point */
 };
 
 const char* xfc_strerror(int code);
@@ -106,6 +107,24 @@ int xfc_fwd_grad_coo(const void* X, int64_t ldx, const void* W, int64_t ldw,
                      const int64_t* pos_x, const int64_t* pos_y, int64_t nnz,
                      void* G, int64_t ldg, int64_t B, int64_t L, int64_t d,
                      float* loss, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * xfc_fwd_grad_csr for callers that cannot allocate device memory or hand over a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results as xfc_fwd_grad_csr minus the workspace: the label buckets
+ * live in a fixed XFC_STATIC_SCRATCH_BYTES array inside the library's device image (one copy per GPU,
+ * held until the process ends), and the call makes no hipMalloc / hipFree.  Problems whose bucket
+ * tables do not fit (xfc_fwd_grad_workspace_bytes(L, nnz) > XFC_STATIC_SCRATCH_BYTES, i.e. beyond
+ * about 16.7 M labels with 190 k positives) are rejected with XFC_ERR_LIMIT.  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;
+ * calls in sequence are independent, every table being rebuilt from scratch by each call.
+ * Call xfc_init() once per device beforehand (it looks the array's device address up).
+ */
+#define XFC_STATIC_SCRATCH_BYTES (2 * 1024 * 1024)
+int xfc_fwd_grad_csr_static(const void* X, int64_t ldx, const void* W, int64_t ldw,
+                            const int32_t* rowptr, const int32_t* colidx,
+                            void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, int64_t nnz,
+                            float* loss, void* stream);
 
 /*
  * dX[B x d] (fp32) = scale * G[B x L] . W[L x d].

@@ -23,6 +23,7 @@ _SIGNATURES = {
     "xfc_logits": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp]),
     "xfc_fwd_grad_workspace_bytes": (_sz, [_i64, _i64]),
     "xfc_fwd_grad_csr": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _sz, _vp]),
+    "xfc_fwd_grad_csr_static": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
     "xfc_fwd_grad_coo": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _sz, _vp]),
     "xfc_dx_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "xfc_dx": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),

@@ -914,6 +914,10 @@ __global__ void __launch_bounds__(256) sgd_momentum_kernel(half_t* __restrict__ 
 
 }  // namespace xfc
 
+// Scratch of xfc_fwd_grad_csr_static: one copy per GPU, held until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress; kernels get the per-device address it returns.
+static __device__ __align__(256) unsigned char g_static_scratch[XFC_STATIC_SCRATCH_BYTES];
+
 // =============================================================================================
 // C ABI
 // =============================================================================================
@@ -975,6 +979,23 @@ int num_cus() {
     n[dev].store(v, std::memory_order_relaxed);
   }
   return v;
+}
+
+// Device address of g_static_scratch on the current device (each GPU holds its own copy at its own
+// address), looked up once per device; nullptr with the error printed if the lookup fails.
+void* static_scratch_ptr() {
+  static std::atomic<void*> ptr[MAX_DEVICES];
+  const int dev = current_device();
+  void* p = ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess || p == nullptr) {
+      fprintf(stderr, "xfc: hipGetSymbolAddress(static scratch) failed: %s\n", hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr[dev].store(p, std::memory_order_release);
+  }
+  return p;
 }
 
 constexpr size_t LOSS_PART_BYTES = 4096;  // one float per forward workgroup (at most 1024)
@@ -1113,6 +1134,7 @@ const char* xfc_strerror(int code) {
     case XFC_ERR_WORKSPACE: return "workspace missing or too small";
     case XFC_ERR_HIP: return "HIP runtime error";
     case XFC_ERR_SHAPE: return "operand shapes do not agree";
+    case XFC_ERR_LIMIT: return "problem larger than the fixed capacity of this entry point";
     default: return "unknown error";
   }
 }
@@ -1133,6 +1155,7 @@ int xfc_init(void) {
   keep(raise_lds_limit<dw_kernel<DW_OUT>>(DW_LDS_BYTES));
   keep(raise_lds_limit<topk_kernel>(TOPK_LDS_BYTES));
   (void)num_cus();
+  if (static_scratch_ptr() == nullptr) return XFC_ERR_HIP;
   if (e != hipSuccess) {
     fprintf(stderr, "xfc: xfc_init failed: %s\n", hipGetErrorString(e));
     return XFC_ERR_HIP;
@@ -1252,6 +1275,25 @@ int xfc_fwd_grad_csr(const void* X, int64_t ldx, const void* W, int64_t ldw, con
   if (B > 0 && !rowptr) return XFC_ERR_INVALID;
   return fwd_grad_impl(X, ldx, W, ldw, rowptr, colidx, nullptr, nullptr, nnz, G, ldg, B, L, d, loss, workspace,
                        workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_fwd_grad_csr_static(const void* X, int64_t ldx, const void* W, int64_t ldw, const int32_t* rowptr,
+                            const int32_t* colidx, void* G, int64_t ldg, int64_t B, int64_t L, int64_t d, int64_t nnz,
+                            float* loss, void* stream) {
+  if (B > 0 && !rowptr) return XFC_ERR_INVALID;
+  if (!dims_ok(L) || nnz < 0) return XFC_ERR_INVALID;
+  if (bucket_ws_bytes(L, nnz) > (size_t)XFC_STATIC_SCRATCH_BYTES) {
+    fprintf(stderr, "xfc_fwd_grad_csr_static: L = %lld labels with %lld positives need %zu bytes of scratch, the static "
+                    "buffer holds %d; use xfc_fwd_grad_csr with a caller workspace\n",
+            (long long)L, (long long)nnz, bucket_ws_bytes(L, nnz), XFC_STATIC_SCRATCH_BYTES);
+    return XFC_ERR_LIMIT;
+  }
+  void* scratch = static_scratch_ptr();
+  if (scratch == nullptr) return XFC_ERR_HIP;
+  // every table in the scratch is rebuilt from its first entry by the bucket pass, so nothing of the
+  // previous call's contents survives into this one
+  return fwd_grad_impl(X, ldx, W, ldw, rowptr, colidx, nullptr, nullptr, nnz, G, ldg, B, L, d, loss, scratch,
+                       (size_t)XFC_STATIC_SCRATCH_BYTES, reinterpret_cast<hipStream_t>(stream));
 }
 
 int xfc_fwd_grad_coo(const void* X, int64_t ldx, const void* W, int64_t ldw, const int64_t* pos_x, const int64_t* pos_y,
