@@ -116,22 +116,31 @@ __device__ __forceinline__ int kc_swz(int row) {
 // transposing read touches then sit in four different 64-byte bank groups.
 __device__ __forceinline__ int mc_swz(int k) { return (k & 3) << 2; }
 
+// FETCH_WAVES_: how many of the workgroup's waves issue the global->LDS fetches (the first FETCH_WAVES_ wave
+// ids; 0 = all).  The fetch path of a CU accepts about 1 KB per 9 ns, so the fetches of one 64 KB stage keep the
+// waves that issue them waiting for 700-1200 cycles (shader-clock marks around the burst); a wave waiting there
+// issues no MFMA.  A fetch in the scalar-base form does not slow the MFMAs of another wave on the same SIMD
+// (3 ns per fetch in a microbenchmark), so with only the first half of the waves fetching -- a workgroup's
+// waves are dealt round-robin over the four SIMDs, which makes that one wave per SIMD -- the other wave of each
+// SIMD multiplies through the burst: 3-5 % on the forward and dX kernels.
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool A_KC_, bool B_KC_, bool ACC_AGPR_ = false,
-          bool A_NT_ = false, bool B_NT_ = false>
+          bool A_NT_ = false, bool B_NT_ = false, int FETCH_WAVES_ = 0>
 struct PipeCore {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, STAGES = STAGES_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
   static constexpr int NW = WM * WN, NT = 64 * NW;
+  static constexpr int NWF = FETCH_WAVES_ > 0 ? FETCH_WAVES_ : NW;  // waves that fetch
   static constexpr int TM = BM / WM, TN = BN / WN;
   static constexpr int FM = TM / 32, FN = TN / 32;
   static constexpr int CPR = BK / 8;
   static constexpr int A_HALVES = BM * BK, B_HALVES = BN * BK;
   static constexpr int STAGE_HALVES = A_HALVES + B_HALVES;
   static constexpr int LDS_BYTES = STAGES * STAGE_HALVES * 2;
-  static constexpr int A_CH = BM * BK / 8 / NT, B_CH = BN * BK / 8 / NT;
-  static constexpr int LOADS_PER_STAGE = A_CH + B_CH;
+  static constexpr int A_CH = BM * BK / 8 / (64 * NWF), B_CH = BN * BK / 8 / (64 * NWF);
+  static constexpr int LOADS_PER_STAGE = A_CH + B_CH;  // per fetching wave
   static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile must be 32-multiples");
-  static_assert((BM * BK / 8) % NT == 0 && (BN * BK / 8) % NT == 0, "chunk split");
+  static_assert((BM * BK / 8) % (64 * NWF) == 0 && (BN * BK / 8) % (64 * NWF) == 0, "chunk split");
+  static_assert(NWF <= NW && NWF % 2 == 0, "fetching waves");
   static_assert(BK == 32 || BK == 64, "BK");
   static_assert(A_KC || BM >= 128, "MC swizzle needs 16 chunks per k-row");
   static_assert(B_KC || BN >= 128, "MC swizzle needs 16 chunks per k-row");
@@ -171,11 +180,11 @@ struct PipeCore {
       if constexpr (KC) {
         kstep = (int64_t)BK * 2;
         kbytes = uniform64((int64_t)k_begin * 2);
-        const int c = pc ^ kc_swz<BK>(wave * RPI + sub);  // the swizzle does not depend on i (NW is even)
+        const int c = pc ^ kc_swz<BK>(wave * RPI + sub);  // the swizzle does not depend on i (NWF is even)
         kin = c * 8;
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
-          const int row0 = o.r0 + (i * NW + wave) * RPI;
+          const int row0 = o.r0 + (i * NWF + wave) * RPI;
           const int g = row0 < o.rmax ? row0 : o.rmax - 1;
           const int row = row0 + sub < o.rmax ? row0 + sub : o.rmax - 1;
           grp[i] = uniform64((int64_t)g * o.ld * 2);
@@ -190,7 +199,7 @@ struct PipeCore {
         kin = sub;
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
-          kgrp[i] = (i * NW + wave) * RPI;
+          kgrp[i] = (i * NWF + wave) * RPI;
           grp[i] = uniform64((int64_t)kgrp[i] * o.ld * 2);
           voff[i] = (uint32_t)sub * (uint32_t)(o.ld * 2) + (uint32_t)col * 2u;
         }
@@ -201,13 +210,13 @@ struct PipeCore {
       if (k0 + BK <= kmax) {
 #pragma unroll
         for (int i = 0; i < CH; ++i)
-          load16_to_lds<NT>(base + grp[i] + kbytes, voff[i], region + (i * NW + wave) * 512);
+          load16_to_lds<NT>(base + grp[i] + kbytes, voff[i], region + (i * NWF + wave) * 512);
       } else {  // the stage that crosses kmax: pieces past it come from the block of zeros
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
           const bool valid = k0 + kgrp[i] + kin < kmax;
           const void* src = valid ? (const void*)(base + grp[i] + kbytes + voff[i]) : (const void*)g_zero16;
-          load16_to_lds<NT>(src, region + (i * NW + wave) * 512);
+          load16_to_lds<NT>(src, region + (i * NWF + wave) * 512);
         }
       }
       kbytes += kstep;
@@ -329,11 +338,14 @@ struct PipeCore {
       la.init(oa, i_k, wave, lane);
       lb.init(ob, i_k, wave, lane);
     }
+    const bool fetcher = wave < NWF;  // wave-uniform
     auto issue_one = [&]() {
       half_t* st = lds + i_slot * STAGE_HALVES;
       if (i_live) {
-        la.issue(st, i_k, wave);
-        lb.issue(st + A_HALVES, i_k, wave);
+        if (fetcher) {
+          la.issue(st, i_k, wave);
+          lb.issue(st + A_HALVES, i_k, wave);
+        }
         i_k += BK;
         if (i_k >= i_kend) {
           ++i_item;
@@ -346,10 +358,10 @@ struct PipeCore {
             i_live = false;
           }
         }
-      } else {
+      } else if (fetcher) {
         // past the last stage: keep the count of outstanding fetches per iteration constant
 #pragma unroll
-        for (int i = 0; i < LOADS_PER_STAGE; ++i) load16_to_lds((const void*)g_zero16, 0u, st + (i * NW + wave) * 512);
+        for (int i = 0; i < LOADS_PER_STAGE; ++i) load16_to_lds((const void*)g_zero16, 0u, st + (i * NWF + wave) * 512);
       }
       i_slot = i_slot + 1 == STAGES ? 0 : i_slot + 1;
     };

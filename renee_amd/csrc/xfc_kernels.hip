@@ -107,7 +107,7 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
 // ---------------------------------------------------------------------------------------------
 enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2, FWD_SIGMOID_PLAIN = 3 };  // PLAIN: alpha 1, beta 0
 
-using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true>;
+using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true, false, false, false, 4>;  // one wave per SIMD fetches
 // beside the ring: the tile's positives bitmap, later reused as store staging (8 rows x TN labels per wave)
 constexpr int FWD_STG_HALVES = 8 * FwdCore::TN;
 constexpr int FWD_BITMAP_BYTES = FwdCore::BN * (FwdCore::BM / 32) * 4;
@@ -654,7 +654,7 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
 // ---------------------------------------------------------------------------------------------
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
-using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, true>;  // accumulators in AGPRs
+using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, true, false, false, 4>;  // accumulators in AGPRs; one wave per SIMD fetches
 constexpr int DX_LDS_BYTES = DxCore::LDS_BYTES;
 
 struct DxArgs {

@@ -225,7 +225,8 @@ def _pipecore_instantiations():
     for name, args in re.findall(r"using\s+(\w+)\s*=\s*PipeCore<([^>]*)>", src):
         v = [a.strip() for a in args.split(",")]
         bm, bn, bk, wm, wn, stages = (int(x) for x in v[:6])
-        loads = (bm * bk // 8 + bn * bk // 8) // (64 * wm * wn)
+        fetch_waves = int(v[11]) if len(v) > 11 and int(v[11]) > 0 else wm * wn   # waves that issue the fetches
+        loads = (bm * bk // 8 + bn * bk // 8) // (64 * fetch_waves)               # per fetching wave
         found[name] = (stages, loads)
     return found
 
