@@ -154,6 +154,21 @@ int xfc_dw_update(const void* G, int64_t ldg, const void* X, int64_t ldx,
                   float* dW_out, int64_t ld_dw, void* stream);
 
 /*
+ * The same pass on fp32 master weights and fp32 momentum, i.e. the reference's own optimizer regime
+ * (xfc_weight is an fp32 parameter, dl_base.py:185; apex FusedSGD keeps fp32 state, main.py:178-179):
+ *   g = dW + weight_decay*W32 ;  M32 = momentum*M32 + g ;  W32 = W32 - lr*M32 ;  W16 = fp16(W32)
+ * W16 is the fp16 copy the forward and dX passes read; the reference makes it with a separate cast of
+ * the whole matrix every step (dl_base.py:562), here it leaves the update's epilogue.  18 bytes per
+ * weight and step against 8 for xfc_dw_update; use it where updates fall below half an fp16 ulp of W
+ * (small learning rates, the tail of a cosine schedule), which fp16-resident weights would drop.
+ */
+int xfc_dw_update_master(const void* G, int64_t ldg, const void* X, int64_t ldx,
+                         float* W32, int64_t ldw32, float* M32, int64_t ldm32, void* W16, int64_t ldw16,
+                         int64_t B, int64_t L, int64_t d,
+                         float lr, float momentum, float weight_decay,
+                         float* dW_out, int64_t ld_dw, void* stream);
+
+/*
  * Split gradient accumulation (dl_base.py:318-340, :623-633):
  *   grad[L x d] (fp32) = G^T . X + beta*grad      beta = 0 first micro-batch, 1 after
  * followed once per step by xfc_sgd_momentum over count = L*d contiguous elements.
@@ -162,6 +177,9 @@ int xfc_dw(const void* G, int64_t ldg, const void* X, int64_t ldx, float* grad, 
            int64_t B, int64_t L, int64_t d, float beta, void* stream);
 int xfc_sgd_momentum(void* W, void* M, const float* grad, int64_t count,
                      float lr, float momentum, float weight_decay, void* stream);
+/* ... and its fp32-master form (W32, M32 updated, W16 = fp16(W32) written), see xfc_dw_update_master. */
+int xfc_sgd_momentum_master(float* W32, float* M32, void* W16, const float* grad, int64_t count,
+                            float lr, float momentum, float weight_decay, void* stream);
 
 /*
  * One whole step for one batch (dl_base.py:303-344 with accum == 1):

@@ -29,6 +29,9 @@ _SIGNATURES = {
     "xfc_dx": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
     "xfc_dw_update": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _f32, _f32,
                              _vp, _i64, _vp]),
+    "xfc_dw_update_master": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _f32, _f32,
+                                    _vp, _i64, _vp]),
+    "xfc_sgd_momentum_master": (_int, [_vp, _vp, _vp, _vp, _i64, _f32, _f32, _f32, _vp]),
     "xfc_dw": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _f32, _vp]),
     "xfc_sgd_momentum": (_int, [_vp, _vp, _vp, _i64, _f32, _f32, _f32, _vp]),
     "xfc_step_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),

@@ -733,7 +733,7 @@ __global__ void __launch_bounds__(256) dx_reduce_kernel(const float* __restrict_
 // ---------------------------------------------------------------------------------------------
 // dW = G^T . X; either written out (fp32, alpha/beta) or consumed by the momentum update
 // ---------------------------------------------------------------------------------------------
-enum DwMode { DW_OUT = 0, DW_UPDATE = 1 };
+enum DwMode { DW_OUT = 0, DW_UPDATE = 1, DW_UPDATE_MASTER = 2 };  // MASTER: fp32 master weights and momentum, fp16 copy of W
 
 using DwCore = PipeCore<128, 256, 32, 2, 2, 2, false, false>;
 constexpr int DW_STAGE_FLOATS = 8 * 64;  // per wave: 8 label rows x 64 dims
@@ -749,6 +749,8 @@ struct DwArgs {
   float* out; int64_t ldo; float alpha, beta;
   // DW_UPDATE
   half_t* Wt; int64_t ldw; half_t* Mo; int64_t ldm; float lr, mu, wd;
+  // DW_UPDATE_MASTER: fp32 master weights and momentum; Wt above receives the fp16 copy of the new weights
+  float* W32; int64_t ldw32; float* M32; int64_t ldm32;
   float* dw_dump; int64_t ld_dump;  // optional copy of dW (may be null)
   int tiles_m, tiles_n, n_ids;      // n_ids = tiles_n * round_up(tiles_m, 8)
 };
@@ -785,10 +787,22 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
     // W and M pieces are fetched DEPTH strips ahead: one strip in flight per wave leaves HBM latency-bound.
     // They are read once per step, hence non-temporal (measured: 3 % off the kernel).
     constexpr int NS = C::FM * 4 * (C::FN / 2);
-    constexpr int DEPTH = 4;
+    constexpr int DEPTH = MODE == DW_UPDATE_MASTER ? 2 : 4;  // the fp32 pieces take twice the registers per strip
     auto strip_row = [&](int s) { return m0 + wm * C::TM + (s / (4 * (C::FN / 2))) * 32 + 8 * ((s / (C::FN / 2)) % 4) + srow; };
     auto strip_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 8; };
     half8 wq[DEPTH], mq[DEPTH];
+    float4v w32q[DEPTH][2], m32q[DEPTH][2];  // DW_UPDATE_MASTER
+    auto fetch32 = [&](int s, float4v (&wv)[2], float4v (&mv)[2]) {
+      int row = strip_row(s), col = strip_col(s);
+      row = row < a.M ? row : a.M - 1;
+      col = col < a.N ? col : a.N - 8;
+      const float* wp = a.W32 + (int64_t)row * a.ldw32 + col;
+      const float* mp = a.M32 + (int64_t)row * a.ldm32 + col;
+      wv[0] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(wp));
+      wv[1] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(wp + 4));
+      mv[0] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(mp));
+      mv[1] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(mp + 4));
+    };
     // unconditional (out-of-range strips read the last valid row / column block and are not stored):
     // straight-line loads let the compiler count exactly how many may stay in flight at each use
     auto fetch = [&](int s, half8& wv, half8& mv) {
@@ -801,6 +815,10 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
     if constexpr (MODE == DW_UPDATE) {
 #pragma unroll
       for (int s = 0; s < DEPTH && s < NS; ++s) fetch(s, wq[s], mq[s]);
+    }
+    if constexpr (MODE == DW_UPDATE_MASTER) {
+#pragma unroll
+      for (int s = 0; s < DEPTH && s < NS; ++s) fetch32(s, w32q[s], m32q[s]);
     }
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -830,6 +848,40 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
           }
           *reinterpret_cast<float4v*>(o) = o0;
           *reinterpret_cast<float4v*>(o + 4) = o1;
+        }
+      } else if constexpr (MODE == DW_UPDATE_MASTER) {
+        // the reference's regime (fp32 parameter and FusedSGD state, dl_base.py:185, main.py:178-179) with the
+        // per-step fp16 cast of W (dl_base.py:562) written from the same pass
+        float4v wv[2] = {w32q[s % DEPTH][0], w32q[s % DEPTH][1]}, mv[2] = {m32q[s % DEPTH][0], m32q[s % DEPTH][1]};
+        if (s + DEPTH < NS) fetch32(s + DEPTH, w32q[s % DEPTH], m32q[s % DEPTH]);
+        if (in) {
+          if (a.dw_dump) {
+            float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
+            *reinterpret_cast<float4v*>(d) = v0;
+            *reinterpret_cast<float4v*>(d + 4) = v1;
+          }
+          half8 w16;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float wf = wv[e >> 2][e & 3];
+            const float gg = g[e] + a.wd * wf;
+            const float mf = a.mu * mv[e >> 2][e & 3] + gg;
+            float wn = wf - a.lr * mf;
+            // the copy is the rounding of the stored fp32 weight, as the reference's cast is (dl_base.py:562):
+            // the empty statement keeps the compiler from fusing the subtraction and the conversion into one
+            // mixed-precision instruction, which would round the exact difference to fp16 in one step
+            asm volatile("" : "+v"(wn));
+            mv[e >> 2][e & 3] = mf;
+            wv[e >> 2][e & 3] = wn;
+            w16[e] = (half_t)wn;
+          }
+          float* wp = a.W32 + (int64_t)row * a.ldw32 + col;
+          float* mp = a.M32 + (int64_t)row * a.ldm32 + col;
+          *reinterpret_cast<float4v*>(mp) = mv[0];
+          *reinterpret_cast<float4v*>(mp + 4) = mv[1];
+          *reinterpret_cast<float4v*>(wp) = wv[0];
+          *reinterpret_cast<float4v*>(wp + 4) = wv[1];
+          *reinterpret_cast<half8*>(a.Wt + (int64_t)row * a.ldw + col) = w16;
         }
       } else {
         half8 wv = wq[s % DEPTH], mv = mq[s % DEPTH];
@@ -910,6 +962,33 @@ __global__ void __launch_bounds__(256) sgd_momentum_kernel(half_t* __restrict__ 
   }
   reinterpret_cast<half8*>(W)[i] = w;
   reinterpret_cast<half8*>(Mo)[i] = m;
+}
+
+// The same on fp32 master weights and momentum, writing the fp16 copy of the new weights as well.
+__global__ void __launch_bounds__(256) sgd_momentum_master_kernel(float* __restrict__ W32, float* __restrict__ M32,
+                                                                  half_t* __restrict__ W16, const float* __restrict__ grad,
+                                                                  int64_t n8, float lr, float mu, float wd) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  float4v w[2] = {reinterpret_cast<float4v*>(W32)[2 * i], reinterpret_cast<float4v*>(W32)[2 * i + 1]};
+  float4v m[2] = {reinterpret_cast<float4v*>(M32)[2 * i], reinterpret_cast<float4v*>(M32)[2 * i + 1]};
+  const float4v g[2] = {reinterpret_cast<const float4v*>(grad)[2 * i], reinterpret_cast<const float4v*>(grad)[2 * i + 1]};
+  half8 h;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float wf = w[e >> 2][e & 3];
+    const float mf = mu * m[e >> 2][e & 3] + g[e >> 2][e & 3] + wd * wf;
+    float wn = wf - lr * mf;
+    asm volatile("" : "+v"(wn));  // the copy is the rounding of the stored fp32 value (see dw_kernel)
+    m[e >> 2][e & 3] = mf;
+    w[e >> 2][e & 3] = wn;
+    h[e] = (half_t)wn;
+  }
+  reinterpret_cast<float4v*>(W32)[2 * i] = w[0];
+  reinterpret_cast<float4v*>(W32)[2 * i + 1] = w[1];
+  reinterpret_cast<float4v*>(M32)[2 * i] = m[0];
+  reinterpret_cast<float4v*>(M32)[2 * i + 1] = m[1];
+  reinterpret_cast<half8*>(W16)[i] = h;
 }
 
 }  // namespace xfc
@@ -1105,6 +1184,8 @@ int launch_dw(int mode, DwArgs a, hipStream_t st) {
   int64_t grid = 2 * (int64_t)round_up(num_cus(), 8);  // two resident workgroups per CU
   if (grid > ids) grid = ids / 8 * 8 > 0 ? ids / 8 * 8 : ids;
   if (mode == DW_UPDATE) return launch_k<dw_kernel<DW_UPDATE>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  if (mode == DW_UPDATE_MASTER)
+    return launch_k<dw_kernel<DW_UPDATE_MASTER>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
   return launch_k<dw_kernel<DW_OUT>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
 }
 
@@ -1153,6 +1234,7 @@ int xfc_init(void) {
   keep(raise_lds_limit<dx_kernel>(DX_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_UPDATE>>(DW_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_OUT>>(DW_LDS_BYTES));
+  keep(raise_lds_limit<dw_kernel<DW_UPDATE_MASTER>>(DW_LDS_BYTES));
   keep(raise_lds_limit<topk_kernel>(TOPK_LDS_BYTES));
   (void)num_cus();
   if (static_scratch_ptr() == nullptr) return XFC_ERR_HIP;
@@ -1336,6 +1418,37 @@ int xfc_dw_update(const void* G, int64_t ldg, const void* X, int64_t ldx, void* 
   a.Wt = (half_t*)W; a.ldw = ldw; a.Mo = (half_t*)Mo; a.ldm = ldm;
   a.lr = lr; a.mu = momentum; a.wd = weight_decay; a.dw_dump = dW_out; a.ld_dump = ld_dw;
   return launch_dw(DW_UPDATE, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_dw_update_master(const void* G, int64_t ldg, const void* X, int64_t ldx, float* W32, int64_t ldw32, float* M32,
+                         int64_t ldm32, void* W16, int64_t ldw16, int64_t B, int64_t L, int64_t d, float lr,
+                         float momentum, float weight_decay, float* dW_out, int64_t ld_dw, void* stream) {
+  if (!dims_ok(B) || !dims_ok(L) || !dims_ok(d)) return XFC_ERR_INVALID;
+  if (L == 0 || d == 0 || B == 0) return XFC_OK;  // an empty batch is not a step
+  if (!G || !X || !W32 || !M32 || !W16) return XFC_ERR_INVALID;
+  if (ldg % 8 || ldx % 8 || ldw16 % 8 || ldw32 % 4 || ldm32 % 4 || d % 8 || !aligned16(G) || !aligned16(X) ||
+      !aligned16(W32) || !aligned16(M32) || !aligned16(W16))
+    return XFC_ERR_ALIGN;
+  if (dW_out && (ld_dw % 4 || !aligned16(dW_out))) return XFC_ERR_ALIGN;
+  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
+  DwArgs a = {};
+  a.G = (const half_t*)G; a.ldg = ldg; a.X = (const half_t*)X; a.ldx = ldx;
+  a.M = (int)L; a.N = (int)d; a.K = (int)B; a.g_cols = (int)round_up(L, 8);
+  a.Wt = (half_t*)W16; a.ldw = ldw16; a.W32 = W32; a.ldw32 = ldw32; a.M32 = M32; a.ldm32 = ldm32;
+  a.lr = lr; a.mu = momentum; a.wd = weight_decay; a.dw_dump = dW_out; a.ld_dump = ld_dw;
+  return launch_dw(DW_UPDATE_MASTER, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+int xfc_sgd_momentum_master(float* W32, float* M32, void* W16, const float* grad, int64_t count, float lr, float momentum,
+                            float weight_decay, void* stream) {
+  if (count < 0) return XFC_ERR_INVALID;
+  if (count == 0) return XFC_OK;
+  if (!W32 || !M32 || !W16 || !grad) return XFC_ERR_INVALID;
+  if (count % 8 || !aligned16(W32) || !aligned16(M32) || !aligned16(W16) || !aligned16(grad)) return XFC_ERR_ALIGN;
+  const int64_t n8 = count / 8;
+  hipLaunchKernelGGL(sgd_momentum_master_kernel, dim3((unsigned)ceil_div(n8, 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), W32, M32, (half_t*)W16, grad, n8, lr, momentum, weight_decay);
+  return check_launch();
 }
 
 int xfc_dw(const void* G, int64_t ldg, const void* X, int64_t ldx, float* grad, int64_t ld_grad, int64_t B, int64_t L,

@@ -161,11 +161,19 @@ class XFCLayer:
     share scratch, so they may run on two streams at once.  One layer's calls
     must stay on one stream at a time.  `max_positives` bounds the label pairs
     of one batch (default 64 per row of max_batch).
+
+    Optimizer state.  By default W and the momentum live in fp16 only (8 bytes
+    of traffic per weight and step); an update smaller than half an fp16 ulp of
+    the weight it applies to is then lost to rounding.  With
+    `master_weights=True` the layer keeps the reference's regime instead, an
+    fp32 `xfc_weight_master` and an fp32 `momentum_buffer` (dl_base.py:185,
+    main.py:178-179), and `xfc_weight` is the fp16 copy of the master that the
+    GEMMs read, rewritten by the update itself (18 bytes per weight and step).
     """
 
     def __init__(self, numy: int, dims: int, max_batch: int, device="cuda:0", lr: float = 0.05,
                  momentum: float = 0.9, weight_decay: float = 0.0, weight: torch.Tensor | None = None,
-                 seed: int = 0, max_positives: int | None = None):
+                 seed: int = 0, max_positives: int | None = None, master_weights: bool = False):
         self.device = torch.device(device)
         _require(self.device.type == "cuda", "XFCLayer needs a GPU device")
         _require(dims % 8 == 0, "dims must be a multiple of 8")
@@ -181,11 +189,21 @@ class XFCLayer:
             for r0 in range(0, self.numy, step):  # N(0, 0.02): dl_base.py:187
                 r1 = min(self.numy, r0 + step)
                 weight[r0:r1] = (torch.randn(r1 - r0, self.dims, generator=g, device=self.device) * 0.02).half()
+            weight_in = weight
         else:
             _require(tuple(weight.shape) == (self.numy, self.dims), "weight shape")
+            weight_in = weight
             weight = weight.to(device=self.device, dtype=torch.float16).contiguous()
+        self.master_weights = bool(master_weights)
+        if self.master_weights:
+            # an fp32 weight handed in (a reference checkpoint's) is kept exactly; the fp16 copy is its rounding
+            self.xfc_weight_master = weight_in.to(device=self.device, dtype=torch.float32).contiguous().clone()
+            weight = self.xfc_weight_master.to(torch.float16)
+            self.momentum_buffer = torch.zeros_like(self.xfc_weight_master)
+        else:
+            self.xfc_weight_master = None
+            self.momentum_buffer = torch.zeros_like(weight)
         self.xfc_weight = weight
-        self.momentum_buffer = torch.zeros_like(self.xfc_weight)
         self.outsoft = torch.empty(self.max_batch, self.ldg, device=self.device, dtype=torch.float16)
         self.grad_input = torch.empty(self.max_batch, self.dims, device=self.device, dtype=torch.float32)
         self.xfc_weight_grad = None  # fp32 accumulator, only under split accumulation
@@ -325,6 +343,16 @@ class XFCLayer:
             _require(dW_out.dtype == torch.float32 and dW_out.is_contiguous() and dW_out.device == self.device and
                      tuple(dW_out.shape) == (self.numy, self.dims),
                      "dW_out must be contiguous float32 (numy, dims) on the layer's device")
+        if self.master_weights:
+            with torch.cuda.device(self.device):
+                rc = lib().xfc_dw_update_master(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0),
+                                                self.xfc_weight_master.data_ptr(), self.dims,
+                                                self.momentum_buffer.data_ptr(), self.dims,
+                                                self.xfc_weight.data_ptr(), self.dims, bsz, self.numy, self.dims,
+                                                self.lr if lr is None else float(lr), self.momentum, self.weight_decay,
+                                                None if dW_out is None else dW_out.data_ptr(), self.dims, _stream(x))
+            check(rc, "xfc_dw_update_master")
+            return
         with torch.cuda.device(self.device):
             rc = lib().xfc_dw_update(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0),
                                      self.xfc_weight.data_ptr(), self.dims, self.momentum_buffer.data_ptr(), self.dims,
@@ -349,6 +377,15 @@ class XFCLayer:
     def optimizer_step(self, lr: float | None = None) -> None:
         """SGD-momentum on the accumulated fp32 grad, then drop it (dl_base.py:343-344)."""
         _require(self.xfc_weight_grad is not None, "no accumulated gradient")
+        if self.master_weights:
+            with torch.cuda.device(self.device):
+                rc = lib().xfc_sgd_momentum_master(self.xfc_weight_master.data_ptr(), self.momentum_buffer.data_ptr(),
+                                                   self.xfc_weight.data_ptr(), self.xfc_weight_grad.data_ptr(),
+                                                   self.numy * self.dims, self.lr if lr is None else float(lr),
+                                                   self.momentum, self.weight_decay, _stream(self.xfc_weight))
+            check(rc, "xfc_sgd_momentum_master")
+            self.xfc_weight_grad = None
+            return
         with torch.cuda.device(self.device):
             rc = lib().xfc_sgd_momentum(self.xfc_weight.data_ptr(), self.momentum_buffer.data_ptr(),
                                         self.xfc_weight_grad.data_ptr(), self.numy * self.dims,
@@ -359,8 +396,10 @@ class XFCLayer:
 
     # -- checkpoint payload (dl_base.py:412-446 keeps xfc_weight and the optimizer state per rank) ------
     def state_dict(self) -> dict:
-        """W and the momentum as CPU fp16 tensors plus the hyper-parameters, for a checkpoint."""
-        return {"xfc_weight": self.xfc_weight.detach().cpu(), "momentum_buffer": self.momentum_buffer.detach().cpu(),
+        """W and the momentum as CPU tensors (fp16, or the fp32 master and momentum when the layer keeps
+        them) plus the hyper-parameters, for a checkpoint."""
+        w = self.xfc_weight_master if self.master_weights else self.xfc_weight
+        return {"xfc_weight": w.detach().cpu(), "momentum_buffer": self.momentum_buffer.detach().cpu(),
                 "numy": self.numy, "dims": self.dims, "lr": self.lr, "momentum": self.momentum,
                 "weight_decay": self.weight_decay}
 
@@ -373,7 +412,11 @@ class XFCLayer:
         first step does."""
         w = state["xfc_weight"]
         _require(tuple(w.shape) == (self.numy, self.dims), "checkpoint shape does not match this layer")
-        self.xfc_weight.copy_(w.to(device=self.device, dtype=torch.float16))
+        if self.master_weights:
+            self.xfc_weight_master.copy_(w.to(device=self.device, dtype=torch.float32))
+            self.xfc_weight.copy_(self.xfc_weight_master)
+        else:
+            self.xfc_weight.copy_(w.to(device=self.device, dtype=torch.float16))
         m = state.get("momentum_buffer")
         if m is None and optimizer_state is not None:
             per_param = list(optimizer_state.get("state", {}).values())
@@ -384,7 +427,7 @@ class XFCLayer:
             self.momentum_buffer.zero_()
         else:
             _require(tuple(m.shape) == (self.numy, self.dims), "momentum buffer shape does not match this layer")
-            self.momentum_buffer.copy_(m.to(device=self.device, dtype=torch.float16))
+            self.momentum_buffer.copy_(m.to(device=self.device, dtype=self.momentum_buffer.dtype))
         for k in ("lr", "momentum", "weight_decay"):
             if k in state:
                 setattr(self, k, float(state[k]))
@@ -406,7 +449,13 @@ class XFCLayer:
         return gi
 
     def step_csr(self, embed, rowptr, colidx, scale: float = 1.0, lr: float | None = None) -> torch.Tensor:
-        """The whole step through the single C entry point xfc_step_csr."""
+        """The whole step through the single C entry point xfc_step_csr (with fp32 master weights: the
+        same three passes through their own entry points, the update being xfc_dw_update_master)."""
+        if self.master_weights:
+            self.fwd_grad(embed, rowptr=rowptr, colidx=colidx)
+            gi = self.dx(embed.shape[0], None, scale)
+            self.dw_update(embed, lr=lr)
+            return gi
         x = self._x16(embed)
         bsz = x.shape[0]
         G = self._g_view(bsz)

@@ -438,3 +438,43 @@ def test_empty_batch_and_reference_optimizer_state(dev):
     lay.load_state_dict({"xfc_weight": W.float()},
                         optimizer_state={"state": {0: {"momentum_buffer": m32}}, "param_groups": [{"lr": 0.05}]})
     assert torch.equal(lay.momentum_buffer.cpu(), m32.half())
+
+
+@pytest.mark.parametrize("B,L,d,wd", [(256, 4097, 768, 0.0), (100, 3001, 64, 1e-3)])
+def test_master_weights_update_matches_fp32_oracle(dev, B, L, d, wd):
+    """xfc_dw_update_master: the reference's optimizer regime (fp32 W and momentum, dl_base.py:185,
+    main.py:178-179) with the fp16 copy of W written by the same pass; two steps, then the split
+    accumulation path (xfc_dw + xfc_sgd_momentum_master)."""
+    X, W, P = _problem(B, L, d, seed=51)
+    W32 = synth.make_W(L, d, 51)                    # an fp32 weight that is not fp16-representable
+    px, py = P.coo()
+    Xd = X.to(dev)
+    lay = XFCLayer(L, d, B, dev, lr=0.01, momentum=0.9, weight_decay=wd, weight=W32, master_weights=True)
+    assert torch.equal(lay.xfc_weight_master.cpu(), W32) and torch.equal(lay.xfc_weight.cpu(), W32.half())
+    Wo, Mo = W32.clone(), torch.zeros(L, d)
+    for s in range(2):
+        print(f"master step {s}: B={B} L={L} d={d}", flush=True)
+        G = lay.fwd_grad(Xd, px, py)
+        Gref = O.grad_logits(O.logits(X.float(), Wo.half().float()), px, py)
+        assert rel(G, Gref) <= TOL
+        dW = torch.empty(L, d, device=dev, dtype=torch.float32)
+        lay.dw_update(Xd, dW_out=dW)
+        # the oracle is fed the device's own fp16 G so that only the update is compared
+        Gd = lay.outsoft[:B, :L].float().cpu()
+        dWo = O.dw(Gd, X.float())
+        assert rel(dW, dWo) <= TOL
+        Wn, Mn = O.sgd_momentum(Wo, Mo, dW.cpu(), 0.01, 0.9, wd)
+        assert rel(lay.xfc_weight_master, Wn) <= 1e-6 and rel(lay.momentum_buffer, Mn) <= 1e-6
+        assert torch.equal(lay.xfc_weight, lay.xfc_weight_master.half())
+        Wo, Mo = lay.xfc_weight_master.cpu().clone(), lay.momentum_buffer.cpu().clone()
+    # split accumulation: two micro-batches, then one optimizer step on the fp32 state
+    half = B // 2 // 8 * 8 or B
+    lay.fwd_grad(Xd[:half], *[t[px < half] for t in (px, py)])
+    lay.dw_accumulate(Xd[:half])
+    acc = lay.xfc_weight_grad.clone()
+    lay.optimizer_step()
+    Wn, Mn = O.sgd_momentum(Wo, Mo, acc.cpu(), 0.01, 0.9, wd)
+    assert rel(lay.xfc_weight_master, Wn) <= 1e-6 and rel(lay.momentum_buffer, Mn) <= 1e-6
+    assert torch.equal(lay.xfc_weight, lay.xfc_weight_master.half())
+    st = lay.state_dict()
+    assert st["xfc_weight"].dtype == torch.float32 and st["momentum_buffer"].dtype == torch.float32
