@@ -10,7 +10,7 @@ LIB_NAME = "libxfc_mi355x.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = [os.path.join(HERE, "csrc", "xfc_kernels.hip")]
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-shared",
     # packed-fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # the global->LDS fetches list M0 as clobbered on purpose; hipcc notes that the register is reserved

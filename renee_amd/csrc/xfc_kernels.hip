@@ -107,14 +107,24 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
 // ---------------------------------------------------------------------------------------------
 enum FwdMode { FWD_LINEAR = 0, FWD_SIGMOID = 1, FWD_GRAD = 2, FWD_SIGMOID_PLAIN = 3 };  // PLAIN: alpha 1, beta 0
 
+// Three row-tile heights: 256 rows for training batches, 128 and 64 for small batches (the reference's
+// B = 32 plumbing case, --accum micro-batches, the last partial batch of an epoch), where a 256-row tile
+// would spend most of its MFMAs on padding.  The label tile is 256 wide in all of them (it is also the
+// width of the positives' buckets).  The smaller tiles leave room for a third ring slot.
 using FwdCore = PipeCore<256, 256, 64, 2, 4, 2, true, true, false, false, false, 4>;  // one wave per SIMD fetches
+using FwdCore128 = PipeCore<128, 256, 64, 2, 4, 3, true, true, false, false, false, 4>;
+using FwdCore64 = PipeCore<64, 256, 64, 2, 4, 3, true, true, false, false, false, 4>;
 // beside the ring: the tile's positives bitmap, later reused as store staging (8 rows x TN labels per wave)
-constexpr int FWD_STG_HALVES = 8 * FwdCore::TN;
-constexpr int FWD_BITMAP_BYTES = FwdCore::BN * (FwdCore::BM / 32) * 4;
-constexpr int FWD_AUX_BYTES = FWD_BITMAP_BYTES > FwdCore::NW * FWD_STG_HALVES * 2 ? FWD_BITMAP_BYTES
-                                                                                    : FwdCore::NW * FWD_STG_HALVES * 2;
-static_assert(FwdCore::FN % 2 == 0, "staging read-back walks 64-label pieces");
-constexpr int FWD_LDS_BYTES = FwdCore::LDS_BYTES + FWD_AUX_BYTES;
+template <class C>
+struct FwdLds {
+  static constexpr int STG_HALVES = 8 * C::TN;
+  static constexpr int BITMAP_BYTES = C::BN * (C::BM / 32) * 4;
+  static constexpr int AUX_BYTES = BITMAP_BYTES > C::NW * STG_HALVES * 2 ? BITMAP_BYTES : C::NW * STG_HALVES * 2;
+  static constexpr int BYTES = C::LDS_BYTES + AUX_BYTES;
+  static_assert(C::FN % 2 == 0, "staging read-back walks 64-label pieces");
+  static_assert(C::BN == 256 && C::NT == 512, "bucket width and workgroup size are shared by all row-tile heights");
+  static_assert(BYTES <= 160 * 1024, "LDS budget");
+};
 
 struct FwdArgs {
   const half_t* X; int64_t ldx;     // M x K, K-contiguous
@@ -129,9 +139,9 @@ struct FwdArgs {
 
 // Persistent: workgroup w takes tile ids w, w + gridDim.x, ... (gridDim.x a multiple of 8, so an
 // id keeps its XCD and the row tiles of one label tile run side by side on one L2).
-template <int MODE, bool BETA, bool LOSS = false>
-__global__ void __launch_bounds__(FwdCore::NT) fwd_kernel(FwdArgs a) {
-  using C = FwdCore;
+template <class C, int MODE, bool BETA, bool LOSS = false>
+__global__ void __launch_bounds__(C::NT) fwd_kernel(FwdArgs a) {
+  constexpr int FWD_STG_HALVES = FwdLds<C>::STG_HALVES;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
   // beside the ring: first the tile's positives bitmap, then per-wave store staging
@@ -298,18 +308,19 @@ __global__ void __launch_bounds__(64) loss_reduce_kernel(const float* __restrict
 // is rescanned exactly, eight columns at a time.  A second kernel merges the groups' lists.
 constexpr int TOPK_MAX = 8;
 constexpr int TOPK_CAP = 4;  // filtered candidates a row can take per tile on the fast path
-using TopkCore = FwdCore;
+template <class C>
 struct TopkLds {
-  float list_v[TopkCore::BM][TOPK_MAX];
-  int32_t list_i[TopkCore::BM][TOPK_MAX];
-  float tau[TopkCore::BM];
-  int32_t cnt[TopkCore::BM];
-  float buf_v[TopkCore::BM][TOPK_CAP];  // fast path: candidates; slow path: 8 staged columns (with buf_i)
-  int32_t buf_i[TopkCore::BM][TOPK_CAP];
+  float list_v[C::BM][TOPK_MAX];
+  int32_t list_i[C::BM][TOPK_MAX];
+  float tau[C::BM];
+  int32_t cnt[C::BM];
+  float buf_v[C::BM][TOPK_CAP];  // fast path: candidates; slow path: 8 staged columns (with buf_i)
+  int32_t buf_i[C::BM][TOPK_CAP];
   int32_t overflow;
+  static constexpr int BYTES = C::LDS_BYTES + (int)(sizeof(float) * C::BM * (2 * TOPK_MAX + 2 + 2 * TOPK_CAP) + 16);
 };
-constexpr int TOPK_LDS_BYTES = TopkCore::LDS_BYTES + (int)sizeof(TopkLds);
-static_assert(TOPK_LDS_BYTES <= 160 * 1024, "top-K LDS budget");
+static_assert(TopkLds<FwdCore>::BYTES <= 160 * 1024 && TopkLds<FwdCore128>::BYTES <= 160 * 1024 &&
+              TopkLds<FwdCore64>::BYTES <= 160 * 1024, "top-K LDS budget");
 static_assert(2 * TOPK_CAP == 8, "the exact rescan stages 8 columns in the candidate buffers");
 
 struct TopkArgs {
@@ -338,17 +349,18 @@ __device__ __forceinline__ void topk_insert(float* lv, int32_t* li, int K, float
 
 // Out of line on purpose: inlined 128 times into the filter, the bodies get merged by the compiler and
 // the register pressure of the whole epilogue explodes (about 180 spilled registers against 2).
-__device__ __attribute__((noinline)) void topk_push(TopkLds& S, int row, float v, int col) {
+template <class S_t>
+__device__ __attribute__((noinline)) void topk_push(S_t& S, int row, float v, int col) {
   const int slot = atomicAdd(&S.cnt[row], 1);
   if (slot < TOPK_CAP) { S.buf_v[row][slot] = v; S.buf_i[row][slot] = col; }
   else S.overflow = 1;
 }
 
-__global__ void __launch_bounds__(TopkCore::NT) topk_kernel(TopkArgs a) {
-  using C = TopkCore;
+template <class C>
+__global__ void __launch_bounds__(C::NT) topk_kernel(TopkArgs a) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
-  TopkLds& S = *reinterpret_cast<TopkLds*>(smem_raw + C::LDS_BYTES);
+  TopkLds<C>& S = *reinterpret_cast<TopkLds<C>*>(smem_raw + C::LDS_BYTES);
   // ids are dealt round-robin to XCDs: the row tiles of one label group sit side by side on one XCD
   int mt, grp;
   xcd_map(blockIdx.x, a.tiles_m, mt, grp);
@@ -655,7 +667,8 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
 // dX = alpha * G . W (+ beta * dX): split over the label axis, fp32 partials, then a reduce
 // ---------------------------------------------------------------------------------------------
 using DxCore = PipeCore<256, 256, 64, 2, 4, 2, true, false, true, false, false, 4>;  // accumulators in AGPRs; one wave per SIMD fetches
-constexpr int DX_LDS_BYTES = DxCore::LDS_BYTES;
+using DxCore128 = PipeCore<128, 256, 64, 2, 4, 3, true, false, true, false, false, 4>;  // small batches, as in the forward pass
+using DxCore64 = PipeCore<64, 256, 64, 2, 4, 3, true, false, true, false, false, 4>;
 
 struct DxArgs {
   const half_t* G; int64_t ldg;   // M x K, K-contiguous (K = labels)
@@ -666,8 +679,8 @@ struct DxArgs {
 };
 
 // One workgroup per (output tile, slice of the label axis); the tiles of one slice get ids on one XCD.
-__global__ void __launch_bounds__(DxCore::NT) dx_kernel(DxArgs a) {
-  using C = DxCore;
+template <class C>
+__global__ void __launch_bounds__(C::NT) dx_kernel(DxArgs a) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
   int tile, split;
@@ -1101,6 +1114,34 @@ BucketWs carve_bucket_ws(void* ws, int64_t L, int64_t nnz) {
   return b;
 }
 
+// Row-tile height for a batch of M rows (see FwdCore / FwdCore128 / FwdCore64).
+inline int row_tile(int64_t M) { return M <= 64 ? 64 : M <= 128 ? 128 : 256; }
+
+template <class C>
+int launch_fwd_c(int mode, FwdArgs a, hipStream_t st, float* loss_part, float* loss_out) {
+  constexpr int LDS = FwdLds<C>::BYTES;
+  a.tiles_m = ceil_div(a.M, C::BM);
+  a.tiles_n = ceil_div(a.n_store, C::BN);
+  const int64_t ids = (int64_t)a.tiles_m * round_up(a.tiles_n, 8);
+  if (ids <= 0) return XFC_OK;
+  if (ids > 0x7fffffff) return XFC_ERR_INVALID;
+  a.n_ids = (int)ids;
+  int64_t grid = (int64_t)round_up(num_cus(), 8);  // one resident workgroup per CU
+  if (grid > ids) grid = ids;                    // ids is a multiple of 8
+  dim3 g((unsigned)grid), b(C::NT);
+  if (mode == FWD_GRAD && loss_part) {
+    int rc = launch_k<fwd_kernel<C, FWD_GRAD, false, true>>(g, b, LDS, st, a);
+    if (rc) return rc;
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(64), 0, st, loss_part, (int)grid, loss_out);
+    return check_launch();
+  }
+  if (mode == FWD_GRAD) return launch_k<fwd_kernel<C, FWD_GRAD, false>>(g, b, LDS, st, a);
+  if (mode == FWD_SIGMOID && a.beta != 0.f) return launch_k<fwd_kernel<C, FWD_SIGMOID, true>>(g, b, LDS, st, a);
+  if (mode == FWD_SIGMOID && a.alpha == 1.0f) return launch_k<fwd_kernel<C, FWD_SIGMOID_PLAIN, false>>(g, b, LDS, st, a);
+  if (mode == FWD_SIGMOID) return launch_k<fwd_kernel<C, FWD_SIGMOID, false>>(g, b, LDS, st, a);
+  return launch_k<fwd_kernel<C, FWD_LINEAR, false>>(g, b, LDS, st, a);
+}
+
 int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, half_t* out, int64_t ldo, int M,
                int N, int K, int n_store, float alpha, float beta, const BucketWs* bk, hipStream_t st,
                float* loss_part = nullptr, float* loss_out = nullptr) {
@@ -1111,40 +1152,29 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
   a.ent_row = bk ? bk->ent_row : nullptr;
   a.ent_col = bk ? bk->ent_col : nullptr;
   a.loss_part = loss_part;
-  a.tiles_m = ceil_div(M, FwdCore::BM);
-  a.tiles_n = ceil_div(n_store, FwdCore::BN);
-  const int64_t ids = (int64_t)a.tiles_m * round_up(a.tiles_n, 8);
-  if (ids <= 0) return XFC_OK;
-  if (ids > 0x7fffffff) return XFC_ERR_INVALID;
-  a.n_ids = (int)ids;
-  int64_t grid = (int64_t)round_up(num_cus(), 8);  // one resident workgroup per CU
-  if (grid > ids) grid = ids;                    // ids is a multiple of 8
-  dim3 g((unsigned)grid), b(FwdCore::NT);
-  if (mode == FWD_GRAD && loss_part) {
-    int rc = launch_k<fwd_kernel<FWD_GRAD, false, true>>(g, b, FWD_LDS_BYTES, st, a);
-    if (rc) return rc;
-    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(64), 0, st, loss_part, (int)grid, loss_out);
-    return check_launch();
+  a.tiles_m = a.tiles_n = a.n_ids = 0;
+  switch (row_tile(M)) {
+    case 64: return launch_fwd_c<FwdCore64>(mode, a, st, loss_part, loss_out);
+    case 128: return launch_fwd_c<FwdCore128>(mode, a, st, loss_part, loss_out);
+    default: return launch_fwd_c<FwdCore>(mode, a, st, loss_part, loss_out);
   }
-  if (mode == FWD_GRAD) return launch_k<fwd_kernel<FWD_GRAD, false>>(g, b, FWD_LDS_BYTES, st, a);
-  if (mode == FWD_SIGMOID && beta != 0.f) return launch_k<fwd_kernel<FWD_SIGMOID, true>>(g, b, FWD_LDS_BYTES, st, a);
-  if (mode == FWD_SIGMOID && alpha == 1.0f) return launch_k<fwd_kernel<FWD_SIGMOID_PLAIN, false>>(g, b, FWD_LDS_BYTES, st, a);
-  if (mode == FWD_SIGMOID) return launch_k<fwd_kernel<FWD_SIGMOID, false>>(g, b, FWD_LDS_BYTES, st, a);
-  return launch_k<fwd_kernel<FWD_LINEAR, false>>(g, b, FWD_LDS_BYTES, st, a);
 }
 
 // Split count for dX: a multiple of 8 slices of the label axis (workgroup ids are dealt round-robin over
 // the 8 XCDs, so the tiles of one slice then meet in one L2), each slice a multiple of the k-step.  The
 // count minimises a cost model fitted to measurements: workgroups run in rounds of one per CU, every
 // workgroup pays a fixed prologue + partial-tile store, and the partial sums are written and read once.
+// A stage of a smaller row tile takes proportionally less time.
 void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& k_per_split) {
-  tiles_m = ceil_div(M, DxCore::BM);
+  const int bm = row_tile(M);
+  tiles_m = ceil_div(M, bm);
   tiles_n = ceil_div(N, DxCore::BN);
   const int64_t tiles = (int64_t)tiles_m * tiles_n > 0 ? (int64_t)tiles_m * tiles_n : 1;
   const int cus = num_cus();
   const double nk = (double)ceil_div(K, DxCore::BK);
   const int max_s = (int)round_up(ceil_div(K, DxCore::BK), 8);
-  constexpr double STAGE_US = 2.4, FIXED_STAGES = 6.0, PART_BYTES_PER_US = 3.0e6;
+  const double STAGE_US = 2.4 * (bm + 256) / 512.0;
+  constexpr double FIXED_STAGES = 6.0, PART_BYTES_PER_US = 3.0e6;
   int best = 8;
   double best_cost = 0.0;
   for (int s = 8; s <= 256 && s <= max_s; s += 8) {
@@ -1166,7 +1196,13 @@ int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float*
   a.M = M; a.N = N; a.K = K;
   const int64_t grid = (int64_t)a.tiles_m * a.tiles_n * a.splits;
   if (grid <= 0 || M <= 0 || N <= 0) return XFC_OK;
-  int rc = launch_k<dx_kernel>(dim3((unsigned)grid), dim3(DxCore::NT), DX_LDS_BYTES, st, a);
+  const dim3 g((unsigned)grid), b(DxCore::NT);
+  int rc;
+  switch (row_tile(M)) {
+    case 64: rc = launch_k<dx_kernel<DxCore64>>(g, b, DxCore64::LDS_BYTES, st, a); break;
+    case 128: rc = launch_k<dx_kernel<DxCore128>>(g, b, DxCore128::LDS_BYTES, st, a); break;
+    default: rc = launch_k<dx_kernel<DxCore>>(g, b, DxCore::LDS_BYTES, st, a); break;
+  }
   if (rc) return rc;
   const int64_t nq = (int64_t)M * (N / 4);
   hipLaunchKernelGGL(dx_reduce_kernel, dim3((unsigned)ceil_div(nq, 256)), dim3(256), 0, st, a.part, out, ldo, M, N,
@@ -1225,17 +1261,25 @@ int xfc_abi_version(void) { return XFC_ABI_VERSION; }
 int xfc_init(void) {
   hipError_t e = hipSuccess;
   auto keep = [&](hipError_t r) { if (e == hipSuccess) e = r; };
-  keep(raise_lds_limit<fwd_kernel<FWD_GRAD, false, true>>(FWD_LDS_BYTES));
-  keep(raise_lds_limit<fwd_kernel<FWD_GRAD, false>>(FWD_LDS_BYTES));
-  keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID, true>>(FWD_LDS_BYTES));
-  keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID, false>>(FWD_LDS_BYTES));
-  keep(raise_lds_limit<fwd_kernel<FWD_SIGMOID_PLAIN, false>>(FWD_LDS_BYTES));
-  keep(raise_lds_limit<fwd_kernel<FWD_LINEAR, false>>(FWD_LDS_BYTES));
-  keep(raise_lds_limit<dx_kernel>(DX_LDS_BYTES));
+  auto fwd_limits = [&](auto core_tag, auto dx_tag) {
+    using C = typename decltype(core_tag)::type;
+    using D = typename decltype(dx_tag)::type;
+    constexpr int LDS = FwdLds<C>::BYTES;
+    keep(raise_lds_limit<fwd_kernel<C, FWD_GRAD, false, true>>(LDS));
+    keep(raise_lds_limit<fwd_kernel<C, FWD_GRAD, false>>(LDS));
+    keep(raise_lds_limit<fwd_kernel<C, FWD_SIGMOID, true>>(LDS));
+    keep(raise_lds_limit<fwd_kernel<C, FWD_SIGMOID, false>>(LDS));
+    keep(raise_lds_limit<fwd_kernel<C, FWD_SIGMOID_PLAIN, false>>(LDS));
+    keep(raise_lds_limit<fwd_kernel<C, FWD_LINEAR, false>>(LDS));
+    keep(raise_lds_limit<topk_kernel<C>>(TopkLds<C>::BYTES));
+    keep(raise_lds_limit<dx_kernel<D>>(D::LDS_BYTES));
+  };
+  fwd_limits(std::type_identity<FwdCore>{}, std::type_identity<DxCore>{});
+  fwd_limits(std::type_identity<FwdCore128>{}, std::type_identity<DxCore128>{});
+  fwd_limits(std::type_identity<FwdCore64>{}, std::type_identity<DxCore64>{});
   keep(raise_lds_limit<dw_kernel<DW_UPDATE>>(DW_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_OUT>>(DW_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_UPDATE_MASTER>>(DW_LDS_BYTES));
-  keep(raise_lds_limit<topk_kernel>(TOPK_LDS_BYTES));
   (void)num_cus();
   if (static_scratch_ptr() == nullptr) return XFC_ERR_HIP;
   if (e != hipSuccess) {
@@ -1501,8 +1545,8 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int
 }
 
 static void topk_plan(int64_t B, int64_t L, int& tiles_m, int& tiles_n, int& n_groups, int& grid) {
-  tiles_m = ceil_div(B, TopkCore::BM);
-  tiles_n = ceil_div(L, TopkCore::BN);
+  tiles_m = ceil_div(B, row_tile(B));
+  tiles_n = ceil_div(L, FwdCore::BN);
   int per = num_cus() / (8 * tiles_m);  // groups per XCD
   if (per < 1) per = 1;
   n_groups = 8 * per;
@@ -1556,7 +1600,13 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   a.cand_v = reinterpret_cast<float*>(workspace);
   a.cand_i = reinterpret_cast<int32_t*>(a.cand_v + (size_t)a.n_groups * B * K);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  int rc = launch_k<topk_kernel>(dim3((unsigned)grid), dim3(TopkCore::NT), TOPK_LDS_BYTES, st, a);
+  const dim3 tg((unsigned)grid), tb(FwdCore::NT);
+  int rc;
+  switch (row_tile(B)) {
+    case 64: rc = launch_k<topk_kernel<FwdCore64>>(tg, tb, TopkLds<FwdCore64>::BYTES, st, a); break;
+    case 128: rc = launch_k<topk_kernel<FwdCore128>>(tg, tb, TopkLds<FwdCore128>::BYTES, st, a); break;
+    default: rc = launch_k<topk_kernel<FwdCore>>(tg, tb, TopkLds<FwdCore>::BYTES, st, a); break;
+  }
   if (rc) return rc;
   hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)B), dim3(64), 0, st, a.cand_v, a.cand_i, (int)B, a.n_groups, K,
                      numy, values, indices);

@@ -478,3 +478,20 @@ def test_master_weights_update_matches_fp32_oracle(dev, B, L, d, wd):
     assert torch.equal(lay.xfc_weight, lay.xfc_weight_master.half())
     st = lay.state_dict()
     assert st["xfc_weight"].dtype == torch.float32 and st["momentum_buffer"].dtype == torch.float32
+
+
+@pytest.mark.parametrize("B", [1, 32, 64, 100, 128, 129])
+def test_small_batches_take_the_small_row_tiles(dev, B):
+    """Batches of up to 64 and up to 128 rows run 64- and 128-row tiles in the forward, dX and top-K kernels
+    (the reference's B = 32 plumbing case, --accum micro-batches dl_base.py:318-340, partial last batches):
+    the whole step and the top-5 against the oracle."""
+    L, d = 5001, 768
+    X, W, P = _problem(B, L, d, kmax=6, kmean=2.0, seed=60 + B)
+    px, py = P.coo()
+    lay = _check_step(dev, X, W, px, py, lr=0.05, mu=0.9, wd=1e-4, scale=4.0, steps=2)
+    v, i = lay.topk(X.to(dev), 5)
+    ov, oi = O.topk(X.float(), lay.xfc_weight.float().cpu(), 5)
+    assert torch.allclose(v.cpu(), ov, rtol=0, atol=1e-3 * float(ov.abs().max()))
+    gap = (ov[:, :-1] - ov[:, 1:]).abs().min(dim=1).values                  # rows whose top-5 is clearly separated
+    sure = gap > 1e-4 * float(ov.abs().max())
+    assert torch.equal(i.cpu()[sure], oi[sure])
