@@ -496,12 +496,13 @@ __global__ void __launch_bounds__(64) topk_merge_kernel(const float* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------
-// top-K for 8 < K <= 128: exact selection over rows of fp16 logits (one workgroup per row)
+// top-K for 8 < K <= 1024: exact selection over rows of fp16 logits (one workgroup per row)
 // ---------------------------------------------------------------------------------------------
-constexpr int SEL_MAX_K = 128;
+constexpr int SEL_MAX_K = 1024;  // one output thread per rank; at most half the sort capacity
 constexpr int SEL_THREADS = 1024;
 constexpr int SEL_BINS = 2048;  // histogram over the top 11 bits of the 16-bit key
 constexpr int SEL_CAP = 2048;   // candidates that are sorted in LDS
+static_assert(SEL_MAX_K <= SEL_THREADS && 2 * SEL_MAX_K <= SEL_CAP, "ranks per row");
 
 // fp16 bit pattern -> 16-bit key that orders like the value (-0 counts as +0).
 __device__ __forceinline__ uint32_t sel_key(uint32_t h) {

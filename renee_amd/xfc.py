@@ -220,9 +220,20 @@ class XFCLayer:
         x = embed.to(device=self.device, dtype=torch.float16)  # dl_base.py:561
         return x if x.stride(1) == 1 and x.stride(0) % 8 == 0 else x.contiguous()
 
-    def _g_view(self, bsz: int) -> torch.Tensor:
-        _require(bsz <= self.max_batch, "batch larger than max_batch")
-        return self.outsoft[0:bsz]
+    def _g_view(self, bsz: int, out: torch.Tensor | None = None) -> torch.Tensor:
+        """The G buffer of a batch: rows of `outsoft`, or a caller's `out` (the reference passes
+        outsoft[0:bsz, :] itself, dl_base.py:312-313) if the kernels can use it as it is: fp16, unit
+        column stride, row stride a multiple of 8 that holds the label count rounded up to 8 (the
+        reference pads numy to a multiple of 16, main.py:83-87)."""
+        if out is None:
+            _require(bsz <= self.max_batch, "batch larger than max_batch")
+            return self.outsoft[0:bsz]
+        _require(out.dtype == torch.float16 and out.dim() == 2 and out.device == self.device and out.stride(1) == 1 and
+                 out.shape[0] == bsz and out.shape[1] in (self.numy, self.ldg) and out.stride(0) % 8 == 0 and
+                 out.stride(0) >= self.ldg and out.data_ptr() % 16 == 0,
+                 "out must be float16 (batch, numy) on the layer's device with a row stride that is a multiple of 8 "
+                 "and at least numy rounded up to 8")
+        return out
 
     def _index(self, t: torch.Tensor, dtype: torch.dtype, what: str) -> torch.Tensor:
         """An index tensor as the kernels read it: 1-D, contiguous, of `dtype`, on this layer's GPU.
@@ -258,12 +269,12 @@ class XFCLayer:
     def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None):
         """Exact top-K labels per row over all labels (FullPredictor's scoring loop, dl_base.py:736-756,
         with the pad clamp of :782 when numy < the stored label count).  Returns (values fp32, indices
-        int64), each (batch, K); ties go to the lower label id.  K <= 128: up to 8 in one fused pass,
+        int64), each (batch, K); ties go to the lower label id.  K <= 1024: up to 8 in one fused pass,
         above that (the final evaluation's K = 100, dl_base.py:817-818) by an exact selection over the
         fp16 logits, which are written to `outsoft` as the reference's scorer does (dl_base.py:745)."""
         x = self._x16(embed)
         bsz = x.shape[0]
-        _require(1 <= K <= 128 and K <= self.numy, "K must be in 1..min(128, numy)")
+        _require(1 <= K <= 1024 and K <= self.numy, "K must be in 1..min(1024, numy)")
         _require(bsz <= self.max_batch, "batch larger than max_batch")
         vals = torch.empty(bsz, K, device=self.device, dtype=torch.float32)
         inds = torch.empty(bsz, K, device=self.device, dtype=torch.int64)
@@ -277,7 +288,7 @@ class XFCLayer:
         return vals, inds
 
     def fwd_grad(self, embed, pos_x=None, pos_y=None, rowptr=None, colidx=None,
-                 loss_out: torch.Tensor | None = None) -> torch.Tensor:
+                 loss_out: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
         """G = sigmoid(embed . W^T) - Y into outsoft (dl_base.py:591-594); returns the (batch, numy) view.
         With loss_out (a one-element float32 tensor) the summed BCE loss of the batch
         (dl_base.py:578-583) is produced by the same pass."""
@@ -287,7 +298,8 @@ class XFCLayer:
         lp = None if loss_out is None else loss_out.data_ptr()
         x = self._x16(embed)
         bsz = x.shape[0]
-        G = self._g_view(bsz)
+        G = self._g_view(bsz, out)
+        ldg = G.stride(0)
         L = lib()
         csr = rowptr is not None
         ws = self._ws
@@ -307,17 +319,18 @@ class XFCLayer:
         with torch.cuda.device(self.device):
             if csr:
                 rc = L.xfc_fwd_grad_csr(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
-                                        rowptr.data_ptr(), colidx.data_ptr(), G.data_ptr(), self.ldg,
+                                        rowptr.data_ptr(), colidx.data_ptr(), G.data_ptr(), ldg,
                                         bsz, self.numy, self.dims, nnz, lp, ws.data_ptr(), ws.numel(), _stream(x))
             else:
                 rc = L.xfc_fwd_grad_coo(x.data_ptr(), x.stride(0), self.xfc_weight.data_ptr(), self.dims,
                                         pos_x.data_ptr() if nnz else None, pos_y.data_ptr() if nnz else None, nnz,
-                                        G.data_ptr(), self.ldg, bsz, self.numy, self.dims, lp,
+                                        G.data_ptr(), ldg, bsz, self.numy, self.dims, lp,
                                         ws.data_ptr(), ws.numel(), _stream(x))
         check(rc, "xfc_fwd_grad")
         return G[:, : self.numy]
 
-    def dx(self, bsz: int, grad_input: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+    def dx(self, bsz: int, grad_input: torch.Tensor | None = None, scale: float = 1.0,
+           out: torch.Tensor | None = None) -> torch.Tensor:
         """grad_input = scale * G . W with W before the update (dl_base.py:602-608)."""
         if grad_input is None:
             grad_input = self.grad_input[0:bsz]
@@ -325,27 +338,29 @@ class XFCLayer:
                  tuple(grad_input.shape) == (bsz, self.dims) and grad_input.device == self.device,
                  "grad_input must be float32 (batch, dims) on the layer's device")
         L = lib()
-        G = self._g_view(bsz)
+        G = self._g_view(bsz, out)
         ws = self._ws
         with torch.cuda.device(self.device):
-            rc = L.xfc_dx(G.data_ptr(), self.ldg, self.xfc_weight.data_ptr(), self.dims, grad_input.data_ptr(),
+            rc = L.xfc_dx(G.data_ptr(), G.stride(0), self.xfc_weight.data_ptr(), self.dims, grad_input.data_ptr(),
                           grad_input.stride(0), bsz, self.numy, self.dims, float(scale),
                           ws.data_ptr(), ws.numel(), _stream(G))
         check(rc, "xfc_dx")
         return grad_input
 
-    def dw_update(self, embed, dW_out: torch.Tensor | None = None, lr: float | None = None) -> None:
+    def dw_update(self, embed, dW_out: torch.Tensor | None = None, lr: float | None = None,
+                  out: torch.Tensor | None = None) -> None:
         """dW = G^T . embed fused with M = mu*M + dW + wd*W ; W -= lr*M (dl_base.py:620-634 + :343)."""
         x = self._x16(embed)
         bsz = x.shape[0]
-        G = self._g_view(bsz)
+        G = self._g_view(bsz, out)
+        ldg = G.stride(0)
         if dW_out is not None:
             _require(dW_out.dtype == torch.float32 and dW_out.is_contiguous() and dW_out.device == self.device and
                      tuple(dW_out.shape) == (self.numy, self.dims),
                      "dW_out must be contiguous float32 (numy, dims) on the layer's device")
         if self.master_weights:
             with torch.cuda.device(self.device):
-                rc = lib().xfc_dw_update_master(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0),
+                rc = lib().xfc_dw_update_master(G.data_ptr(), ldg, x.data_ptr(), x.stride(0),
                                                 self.xfc_weight_master.data_ptr(), self.dims,
                                                 self.momentum_buffer.data_ptr(), self.dims,
                                                 self.xfc_weight.data_ptr(), self.dims, bsz, self.numy, self.dims,
@@ -354,23 +369,23 @@ class XFCLayer:
             check(rc, "xfc_dw_update_master")
             return
         with torch.cuda.device(self.device):
-            rc = lib().xfc_dw_update(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0),
+            rc = lib().xfc_dw_update(G.data_ptr(), ldg, x.data_ptr(), x.stride(0),
                                      self.xfc_weight.data_ptr(), self.dims, self.momentum_buffer.data_ptr(), self.dims,
                                      bsz, self.numy, self.dims, self.lr if lr is None else float(lr), self.momentum,
                                      self.weight_decay, None if dW_out is None else dW_out.data_ptr(), self.dims,
                                      _stream(x))
         check(rc, "xfc_dw_update")
 
-    def dw_accumulate(self, embed) -> None:
+    def dw_accumulate(self, embed, out: torch.Tensor | None = None) -> None:
         """xfc_weight.grad (+)= G^T . embed for one micro-batch (dl_base.py:620-633)."""
         x = self._x16(embed)
         bsz = x.shape[0]
-        G = self._g_view(bsz)
+        G = self._g_view(bsz, out)
         first = self.xfc_weight_grad is None
         if first:
             self.xfc_weight_grad = torch.empty(self.numy, self.dims, device=self.device, dtype=torch.float32)
         with torch.cuda.device(self.device):
-            rc = lib().xfc_dw(G.data_ptr(), self.ldg, x.data_ptr(), x.stride(0), self.xfc_weight_grad.data_ptr(),
+            rc = lib().xfc_dw(G.data_ptr(), G.stride(0), x.data_ptr(), x.stride(0), self.xfc_weight_grad.data_ptr(),
                               self.dims, bsz, self.numy, self.dims, 0.0 if first else 1.0, _stream(x))
         check(rc, "xfc_dw")
 

@@ -495,3 +495,50 @@ def test_small_batches_take_the_small_row_tiles(dev, B):
     gap = (ov[:, :-1] - ov[:, 1:]).abs().min(dim=1).values                  # rows whose top-5 is clearly separated
     sure = gap > 1e-4 * float(ov.abs().max())
     assert torch.equal(i.cpu()[sure], oi[sure])
+
+
+def test_reference_loss_module_interface(dev):
+    """renee_amd.BCELossMultiNode has the reference class's call signature (dl_base.py:576); the XFC
+    block of fit (dl_base.py:303-344) written against it, with the reference's own `out` and
+    `grad_input` views, matches the oracle over two steps, with and without a preceding xfc_forward,
+    the sampled loss on step 0, and under split accumulation."""
+    from renee_amd import BCELossMultiNode
+
+    class Scaler:                       # the part of torch.cuda.amp.GradScaler the path uses (dl_base.py:599)
+        def get_scale(self):
+            return 4096.0
+
+    B, L, d = 96, 4112, 128             # numy padded to a multiple of 16 as main.py:83-87 does
+    X, W, P = _problem(B, L, d, seed=71)
+    z = torch.stack(P.coo())            # the collator's 'z' (2 x nnz LongTensor on the CPU)
+    lay = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W)
+    lm = BCELossMultiNode(lay, compute_loss=True, scaler=Scaler())
+    Wo, Mo = W.float(), torch.zeros(L, d)
+    for step in range(2):
+        embed_out = lm.gather_embed(X.float().to(dev), None)
+        do_forward = step == 0          # a loss step: the reference runs xfc_forward first (dl_base.py:311)
+        out = lay.outsoft[0:B, :]
+        if do_forward:
+            lm.xfc_forward(embed_out, out)
+        loss = lm.xfc_backward(embed_out, out, z[0], z[1], lay.grad_input[0:B, :], not do_forward)
+        lm.xfc_optimizer.step()
+        lm.count += 1
+        ref = O.step(X.float(), Wo, Mo, z[0], z[1], 0.05, 0.9, 0.0, 4096.0)
+        assert rel(lay.grad_input[:B], ref["dX"]) <= TOL
+        assert rel(lay.xfc_weight, ref["W"]) <= TOL and rel(lay.momentum_buffer, ref["M"]) <= TOL
+        if step == 0:
+            want = O.sampled_loss(O.logits(X.float(), Wo), z[0], z[1])
+            assert abs(float(loss) - float(want)) <= 1e-3 * abs(float(want))
+        Wo, Mo = lay.xfc_weight.float().cpu(), lay.momentum_buffer.float().cpu()
+    # --accum 2: two micro-batches into the fp32 grad, then one optimizer step (dl_base.py:318-343)
+    lm2 = BCELossMultiNode(lay, compute_loss=False, scaler=Scaler(), accum=2)
+    half = B // 2
+    idx = [0, int((z[0] < half).sum()), z.shape[1]]
+    for i, (r0, r1) in enumerate(((0, half), (half, B))):
+        e = lm2.gather_embed(X[r0:r1].float().to(dev))
+        lm2.xfc_backward(e, lay.outsoft[0:r1 - r0, :], z[0, idx[i]:idx[i + 1]] - r0, z[1, idx[i]:idx[i + 1]],
+                         lay.grad_input[r0:r1, :], True)
+    lm2.xfc_optimizer.step()
+    ref = O.step(X.float(), Wo, Mo, z[0], z[1], 0.05, 0.9, 0.0, 4096.0)
+    assert rel(lay.grad_input[:B], ref["dX"]) <= TOL
+    assert rel(lay.xfc_weight, ref["W"]) <= TOL and rel(lay.momentum_buffer, ref["M"]) <= TOL

@@ -136,7 +136,8 @@ def _check_select(dev, X, W, K, numy=None, max_ws=None, vs_oracle=True):
 
 
 @pytest.mark.parametrize("B,L,d,K", [(37, 1000, 64, 100), (256, 4096, 768, 100), (64, 70001, 128, 9),
-                                     (5, 128, 8, 128), (3, 100, 8, 100)])
+                                     (5, 128, 8, 128), (3, 100, 8, 100), (9, 5000, 64, 500), (4, 1024, 8, 1024),
+                                     (6, 30000, 32, 1024)])
 def test_topk_select_matches_sort_and_oracle(dev, B, L, d, K):
     X = synth.make_X(B, d, 4).half()
     W = synth.make_W(L, d, 4).half()
