@@ -16,7 +16,9 @@ W moves by O(100 %) per step and MFMA throughput depends on the operand values.
 `ms_per_step` is the mean of the K per-step HIP event intervals; the same K steps
 run back to back without the restore are reported once as `drifting_ms_per_step`.
 The other BASELINE configurations (1, 3 with its top-5 / top-100 scorers, 4) are
-timed the same way with fewer steps and reported under `other_configs`.
+timed the same way with fewer steps and reported under `other_configs`;
+`master_weights` times the update pass with fp32 master weights and momentum, and
+`mfma_power_probe` runs the logits kernel on random and on all-zero operands.
 """
 from __future__ import annotations
 
@@ -180,6 +182,68 @@ def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: boo
     return out
 
 
+def mfma_power_probe(dev):
+    """xfc_logits on cache-resident 4096 x 4096 x 8192 operands, once with random and once with all-zero
+    inputs: the same kernel, instruction stream and memory traffic, so the ratio is what operand
+    switching activity (power) costs the matrix pipes on this chip."""
+    import torch
+
+    from renee_amd import XFCLayer
+
+    B, L, d = 4096, 4096, 8192
+    out = {"shape": f"{B}x{L}x{d} fp16 logits, operands resident in the L2 / Infinity Cache"}
+    lay = XFCLayer(L, d, B, dev)
+    for name in ("random", "zeros"):
+        if name == "zeros":
+            lay.xfc_weight.zero_()
+            X = torch.zeros(B, d, device=dev, dtype=torch.float16)
+        else:
+            X = (torch.randn(B, d, device=dev) * 0.05).half()
+        for _ in range(3):
+            lay.xfc_forward(X)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            lay.xfc_forward(X)
+        e1.record()
+        torch.cuda.synchronize()
+        out[f"{name}_tflops"] = 2.0 * B * L * d / (e0.elapsed_time(e1) / 20 * 1e-3) / 1e12
+    del lay
+    torch.cuda.empty_cache()
+    return out
+
+
+def master_weights_update(cfg: int, seed: int, dev):
+    """The dW + update pass in the reference's optimizer regime (fp32 master weights and momentum, fp16
+    copy of W written by the same pass: 18 bytes per weight) at one configuration."""
+    import torch
+
+    from renee_amd import XFCLayer, synth
+
+    c = synth.CONFIGS[cfg]
+    B, L, d = c["B"], c["L"], synth.D_MODEL
+    lay = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, seed=seed, master_weights=True)
+    X = synth.make_X(B, d, seed, dev).half()
+    P = synth.make_positives(B, L, c["kmax"], c["kmean"], c["zipf"], seed)
+    lay.fwd_grad(X, rowptr=torch.from_numpy(P.rowptr).to(dev), colidx=torch.from_numpy(P.colidx).to(dev))
+    for _ in range(2):
+        lay.dw_update(X, lr=0.0)   # lr 0: the weights stay on the stated distribution, the traffic is the same
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n = 5
+    e0.record()
+    for _ in range(n):
+        lay.dw_update(X, lr=0.0)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / n
+    del lay
+    torch.cuda.empty_cache()
+    return {"dw_update_master_ms": ms, "bytes_per_weight": 18, "gbs": 18.0 * L * d / (ms * 1e-3) / 1e9,
+            "hbm_frac": 18.0 * L * d / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+
 def summarise(r):
     """Per-configuration figures from time_config's result."""
     B, L, d = r["B"], r["L"], r["d"]
@@ -276,6 +340,8 @@ def main() -> int:
                                                               scorers=(cfg == 3)))
             others[f"configs[{cfg}]"]["steps"] = n
         out["other_configs"] = others
+        out["master_weights"] = master_weights_update(args.config, args.seed, dev)
+        out["mfma_power_probe"] = mfma_power_probe(dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.config, d, args.seed)
         out["cpu_baseline_cfg0"] = cpu_baseline_cfg0(d, args.seed)
