@@ -749,9 +749,21 @@ __global__ void __launch_bounds__(256) dx_reduce_kernel(const float* __restrict_
 // ---------------------------------------------------------------------------------------------
 enum DwMode { DW_OUT = 0, DW_UPDATE = 1, DW_UPDATE_MASTER = 2 };  // MASTER: fp32 master weights and momentum, fp16 copy of W
 
-using DwCore = PipeCore<128, 256, 32, 2, 2, 2, false, false>;
+// 256 labels x 256 dims x 64 batch rows per stage, eight waves of 64 labels x 128 dims, one workgroup per CU.
+// (A 128 x 256 x 32 tile with four waves and two workgroups per CU, meant to overlap one workgroup's update with
+// the other's GEMM, measured 7-11 % slower at every batch size: its stages move half again as much through LDS
+// and the fetch path per flop, and the update's streaming is bound by HBM either way.)
+#ifndef XFC_DW_FW
+#define XFC_DW_FW 4
+#endif
+#ifndef XFC_DW_DEPTH
+#define XFC_DW_DEPTH 4
+#endif
+using DwCore = PipeCore<256, 256, 64, 4, 2, 2, false, false, false, false, false, XFC_DW_FW>;
 constexpr int DW_STAGE_FLOATS = 8 * 64;  // per wave: 8 label rows x 64 dims
 constexpr int DW_LDS_BYTES = DwCore::LDS_BYTES + DwCore::NW * DW_STAGE_FLOATS * 4;
+static_assert(DW_LDS_BYTES <= 160 * 1024, "LDS budget");
+static_assert(DwCore::TM == 64 && DwCore::TN == 128, "the update epilogue walks 64 x 128 wave tiles");
 static_assert(DwCore::FN % 2 == 0, "epilogue walks pairs of 32-column blocks");
 
 struct DwArgs {
@@ -769,10 +781,10 @@ struct DwArgs {
   int tiles_m, tiles_n, n_ids;      // n_ids = tiles_n * round_up(tiles_m, 8)
 };
 
-// Persistent, two workgroups per CU: workgroup w takes tile ids w, w + gridDim.x, ...; the dim tiles of
+// Persistent, one workgroup per CU: workgroup w takes tile ids w, w + gridDim.x, ...; the dim tiles of
 // one label tile have neighbouring ids on one XCD, so its slice of G is fetched from HBM once.
 template <int MODE>
-__global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
+__global__ void __launch_bounds__(DwCore::NT) dw_kernel(DwArgs a) {
   using C = DwCore;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
@@ -801,7 +813,7 @@ __global__ void __launch_bounds__(256, 2) dw_kernel(DwArgs a) {
     // W and M pieces are fetched DEPTH strips ahead: one strip in flight per wave leaves HBM latency-bound.
     // They are read once per step, hence non-temporal (measured: 3 % off the kernel).
     constexpr int NS = C::FM * 4 * (C::FN / 2);
-    constexpr int DEPTH = MODE == DW_UPDATE_MASTER ? 2 : 4;  // the fp32 pieces take twice the registers per strip
+    constexpr int DEPTH = MODE == DW_UPDATE_MASTER ? XFC_DW_DEPTH / 2 : XFC_DW_DEPTH;  // the fp32 pieces take twice the registers per strip
     auto strip_row = [&](int s) { return m0 + wm * C::TM + (s / (4 * (C::FN / 2))) * 32 + 8 * ((s / (C::FN / 2)) % 4) + srow; };
     auto strip_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 8; };
     half8 wq[DEPTH], mq[DEPTH];
@@ -1218,12 +1230,12 @@ int launch_dw(int mode, DwArgs a, hipStream_t st) {
   if (ids <= 0) return XFC_OK;
   if (ids > 0x7fffffff) return XFC_ERR_INVALID;
   a.n_ids = (int)ids;
-  int64_t grid = 2 * (int64_t)round_up(num_cus(), 8);  // two resident workgroups per CU
+  int64_t grid = (int64_t)round_up(num_cus(), 8);  // one resident workgroup per CU
   if (grid > ids) grid = ids / 8 * 8 > 0 ? ids / 8 * 8 : ids;
-  if (mode == DW_UPDATE) return launch_k<dw_kernel<DW_UPDATE>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
-  if (mode == DW_UPDATE_MASTER)
-    return launch_k<dw_kernel<DW_UPDATE_MASTER>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
-  return launch_k<dw_kernel<DW_OUT>>(dim3((unsigned)grid), dim3(256), DW_LDS_BYTES, st, a);
+  const dim3 g((unsigned)grid), b(DwCore::NT);
+  if (mode == DW_UPDATE) return launch_k<dw_kernel<DW_UPDATE>>(g, b, DW_LDS_BYTES, st, a);
+  if (mode == DW_UPDATE_MASTER) return launch_k<dw_kernel<DW_UPDATE_MASTER>>(g, b, DW_LDS_BYTES, st, a);
+  return launch_k<dw_kernel<DW_OUT>>(g, b, DW_LDS_BYTES, st, a);
 }
 
 int launch_generic(const void* in1, int64_t as0, int64_t as1, const void* in2, int64_t bs0, int64_t bs1, void* out,
