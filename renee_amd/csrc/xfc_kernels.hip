@@ -753,13 +753,7 @@ enum DwMode { DW_OUT = 0, DW_UPDATE = 1, DW_UPDATE_MASTER = 2 };  // MASTER: fp3
 // (A 128 x 256 x 32 tile with four waves and two workgroups per CU, meant to overlap one workgroup's update with
 // the other's GEMM, measured 7-11 % slower at every batch size: its stages move half again as much through LDS
 // and the fetch path per flop, and the update's streaming is bound by HBM either way.)
-#ifndef XFC_DW_FW
-#define XFC_DW_FW 4
-#endif
-#ifndef XFC_DW_DEPTH
-#define XFC_DW_DEPTH 4
-#endif
-using DwCore = PipeCore<256, 256, 64, 4, 2, 2, false, false, false, false, false, XFC_DW_FW>;
+using DwCore = PipeCore<256, 256, 64, 4, 2, 2, false, false, false, false, false, 4>;
 constexpr int DW_STAGE_FLOATS = 8 * 64;  // per wave: 8 label rows x 64 dims
 constexpr int DW_LDS_BYTES = DwCore::LDS_BYTES + DwCore::NW * DW_STAGE_FLOATS * 4;
 static_assert(DW_LDS_BYTES <= 160 * 1024, "LDS budget");
@@ -813,7 +807,7 @@ __global__ void __launch_bounds__(DwCore::NT) dw_kernel(DwArgs a) {
     // W and M pieces are fetched DEPTH strips ahead: one strip in flight per wave leaves HBM latency-bound.
     // They are read once per step, hence non-temporal (measured: 3 % off the kernel).
     constexpr int NS = C::FM * 4 * (C::FN / 2);
-    constexpr int DEPTH = MODE == DW_UPDATE_MASTER ? XFC_DW_DEPTH / 2 : XFC_DW_DEPTH;  // the fp32 pieces take twice the registers per strip
+    constexpr int DEPTH = MODE == DW_UPDATE_MASTER ? 2 : 4;  // the fp32 pieces take twice the registers per strip (2-6 measure alike)
     auto strip_row = [&](int s) { return m0 + wm * C::TM + (s / (4 * (C::FN / 2))) * 32 + 8 * ((s / (C::FN / 2)) % 4) + srow; };
     auto strip_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 8; };
     half8 wq[DEPTH], mq[DEPTH];
