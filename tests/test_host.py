@@ -307,3 +307,13 @@ def test_main_loop_wait_counts_never_expose_a_stage_in_flight():
     # the model does catch a wait that is one stage too permissive
     for stages, loads in ((3, 8), (4, 4)):
         assert _simulate_ring(stages, loads, [12], 0, slack=loads) != []
+
+
+def test_g_row_stride_is_skewed_off_powers_of_two():
+    from renee_amd.xfc import g_row_stride
+
+    for L in (1310720, 2812281, 16777216, 131072, 131073, 4097):
+        ld = g_row_stride(L)
+        assert ld % 8 == 0 and ld >= (L + 7) // 8 * 8 and ld - L < 2048 + 8
+        assert (ld * 2) % 4096 == 256
+    assert g_row_stride(9) == 16 and g_row_stride(1000) == 1000
