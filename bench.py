@@ -15,8 +15,9 @@ timed step, outside the step's event pair, because at lr = 0.05 on these inputs
 W moves by O(100 %) per step and MFMA throughput depends on the operand values.
 `ms_per_step` is the mean of the K per-step HIP event intervals; the same K steps
 run back to back without the restore are reported once as `drifting_ms_per_step`.
-The other BASELINE configurations (1, 3 with its top-5 / top-100 scorers, 4) are
-timed the same way with fewer steps and reported under `other_configs`;
+The other BASELINE configurations (0 with a batch-256 run at the same label count
+beside it, 1, 3 with its top-5 / top-100 scorers, 4) are timed the same way with
+fewer steps and reported under `other_configs`;
 `master_weights` times the update pass with fp32 master weights and momentum, and
 `mfma_power_probe` runs the logits kernel on random and on all-zero operands.
 """
@@ -100,15 +101,17 @@ def cpu_baseline_cfg0(d: int, seed: int):
             "s_per_step_median": t, "s_per_step_min": ts[0], "gflops": 6.0 * B * L * d / t / 1e9}
 
 
-def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: bool = True, scorers: bool = False):
-    """Times `steps` steps of one BASELINE configuration, each from the same (W0, M1) state."""
+def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: bool = True, scorers: bool = False,
+                batch: int = 0):
+    """Times `steps` steps of one BASELINE configuration (with `batch` rows instead of its own when
+    given), each from the same (W0, M1) state."""
     import torch
 
     from renee_amd import XFCLayer, synth
     from renee_amd._lib import check, lib
 
     c = synth.CONFIGS[cfg]
-    B, L, d = c["B"], c["L"], synth.D_MODEL
+    B, L, d = batch or c["B"], c["L"], synth.D_MODEL
     layer = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight_decay=0.0, seed=seed)
     X = synth.make_X(B, d, seed, dev).half()
     P = synth.make_positives(B, L, c["kmax"], c["kmean"], c["zipf"], seed)
@@ -269,7 +272,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (1..4)")
+    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (0..4)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-others", action="store_true", help="skip the other BASELINE configurations")
     ap.add_argument("--seed", type=int, default=0)
@@ -333,12 +336,16 @@ def main() -> int:
         del src, dst
     if not args.no_others:
         others = {}
-        for cfg, n in ((1, 20), (3, 6), (4, 3)):
+        for cfg, n in ((0, 20), (1, 20), (3, 6), (4, 3)):
             if cfg == args.config:
                 continue
             others[f"configs[{cfg}]"] = summarise(time_config(cfg, n, 2, args.seed, dev, drifting=False,
                                                               scorers=(cfg == 3)))
             others[f"configs[{cfg}]"]["steps"] = n
+        # what the 64-row tiles buy at batch 32: the same label count at batch 256 (one full-height tile)
+        b256 = time_config(0, 20, 2, args.seed, dev, drifting=False, batch=256)["ms_per_step"]
+        others["configs[0]"]["batch256_same_labels_ms_per_step"] = b256
+        others["configs[0]"]["vs_quarter_of_batch256"] = others["configs[0]"]["ms_per_step"] / (b256 / 4.0)
         out["other_configs"] = others
         out["master_weights"] = master_weights_update(args.config, args.seed, dev)
         out["mfma_power_probe"] = mfma_power_probe(dev)
