@@ -306,8 +306,13 @@ __global__ void __launch_bounds__(64) loss_reduce_kernel(const float* __restrict
 // filtered against each row's current K-th score; survivors (few once the lists have warmed up) go to
 // a small per-row buffer that the row's owner thread merges.  If any row overflows its buffer, the tile
 // is rescanned exactly, eight columns at a time.  A second kernel merges the groups' lists.
+// The workgroups that share a row tile also share what they have learnt: each publishes its rows' K-th
+// scores to `bound` (atomic max) and filters against the largest published one as well.  Any published
+// value is the K-th score of K real labels, so nothing below it can be in the row's final list; ties with
+// it pass (a tying label of lower id may still rank above).  This only makes the filter tighter sooner:
+// the lists, and so the results, do not depend on when a bound becomes visible.
 constexpr int TOPK_MAX = 8;
-constexpr int TOPK_CAP = 4;  // filtered candidates a row can take per tile on the fast path
+constexpr int TOPK_CAP = 6;  // filtered candidates a row can take per tile on the fast path (what LDS leaves room for)
 template <class C>
 struct TopkLds {
   float list_v[C::BM][TOPK_MAX];
@@ -321,7 +326,7 @@ struct TopkLds {
 };
 static_assert(TopkLds<FwdCore>::BYTES <= 160 * 1024 && TopkLds<FwdCore128>::BYTES <= 160 * 1024 &&
               TopkLds<FwdCore64>::BYTES <= 160 * 1024, "top-K LDS budget");
-static_assert(2 * TOPK_CAP == 8, "the exact rescan stages 8 columns in the candidate buffers");
+static_assert(2 * TOPK_CAP >= 8, "the exact rescan stages 8 columns in the candidate buffers");
 
 struct TopkArgs {
   const half_t* X; int64_t ldx;
@@ -329,8 +334,25 @@ struct TopkArgs {
   int M, N, K;          // rows, labels, feature dims
   int topk;
   float* cand_v; int32_t* cand_i;  // [n_groups][M][topk]
+  uint32_t* bound;                 // [M] shared lower bounds of the rows' final K-th scores (ordered keys, 0 = none yet)
   int tiles_m, tiles_n, n_groups;
 };
+
+// Floats as unsigned keys in the same order (for atomicMax), and back.
+__device__ __forceinline__ uint32_t topk_key(float f) {
+  const uint32_t b = __float_as_uint(f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float topk_unkey(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+// A value strictly below x (x finite or +inf) and as close to it as a normal number allows: "v > below(x)"
+// admits every v >= x.  Tiny magnitudes step to a fixed small negative so that no denormal is ever compared.
+__device__ __forceinline__ float topk_below(float x) {
+  if (fabsf(x) < 1e-30f) return -1e-30f;
+  const uint32_t b = __float_as_uint(x);
+  return __uint_as_float(x > 0.f ? b - 1u : b + 1u);
+}
 
 __device__ __forceinline__ bool topk_better(float av, int ai, float bv, int bi) {
   return av > bv || (av == bv && ai < bi);
@@ -347,10 +369,10 @@ __device__ __forceinline__ void topk_insert(float* lv, int32_t* li, int K, float
   li[p] = i;
 }
 
-// Out of line on purpose: inlined 128 times into the filter, the bodies get merged by the compiler and
-// the register pressure of the whole epilogue explodes (about 180 spilled registers against 2).
+// Inlined on purpose: a function that is called waits for every outstanding memory operation on entry
+// (the calling convention cannot know what is in flight), which here is the next tile's prefetch.
 template <class S_t>
-__device__ __attribute__((noinline)) void topk_push(S_t& S, int row, float v, int col) {
+__device__ __forceinline__ void topk_push(S_t& S, int row, float v, int col) {
   const int slot = atomicAdd(&S.cnt[row], 1);
   if (slot < TOPK_CAP) { S.buf_v[row][slot] = v; S.buf_i[row][slot] = col; }
   else S.overflow = 1;
@@ -390,6 +412,19 @@ __global__ void __launch_bounds__(C::NT) topk_kernel(TopkArgs a) {
     const int n0 = nt * C::BN;
     const bool ragged = n0 + C::BN > a.N;
     const int h = lane >> 5;
+    // the row owners ask for the shared bound now and use it after the filter
+    const bool owner = threadIdx.x < C::BM && m0 + (int)threadIdx.x < a.M;
+    uint32_t shared_key = 0u;
+    if (owner) shared_key = __hip_atomic_load(a.bound + m0 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // what the filter compares with from the next tile on: the list's K-th score, or just below the shared bound
+    auto settle = [&](int t, bool changed) {
+      const float mine = S.list_v[t][K - 1];
+      if (changed && owner && mine > NEG_INF)
+        __hip_atomic_fetch_max(a.bound + m0 + t, topk_key(mine), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float theirs = shared_key > topk_key(NEG_INF) ? topk_below(topk_unkey(shared_key)) : NEG_INF;
+      S.tau[t] = fmaxf(mine, theirs);
+      S.cnt[t] = 0;
+    };
     // filter against each row's K-th best so far
 #pragma unroll
     for (int fm = 0; fm < C::FM; ++fm) {
@@ -397,14 +432,27 @@ __global__ void __launch_bounds__(C::NT) topk_kernel(TopkArgs a) {
       for (int q = 0; q < 4; ++q) {
         const int row0 = wm * C::TM + fm * 32 + 8 * q + 4 * h;
         const float4v tau4 = *reinterpret_cast<const float4v*>(&S.tau[row0]);
+        // one branch per strip of 4 rows x TN labels: the compares are combined as lane masks, and only a
+        // strip in which some lane holds a survivor walks its elements (rare once the lists have warmed up)
+        bool any = false;
 #pragma unroll
-        for (int fn = 0; fn < C::FN; ++fn) {
-          const int col = n0 + wn * C::TN + fn * 32 + (lane & 31);
-          const bool col_ok = !ragged || col < a.N;
+        for (int fn = 0; fn < C::FN; ++fn)
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            const float v = acc[fm][fn][4 * q + rr];
-            if (v > tau4[rr] && col_ok) topk_push(S, row0 + rr, v, col);  // rare once the lists have warmed up
+          for (int rr = 0; rr < 4; ++rr) any |= acc[fm][fn][4 * q + rr] > tau4[rr];
+        if (__builtin_amdgcn_ballot_w64(any) != 0) {
+          // opaque on purpose: the compiler otherwise computes the list addresses of all 128 elements when
+          // the kernel starts, spills them, and reloads them here behind a wait for every outstanding fetch
+          int r0 = row0;
+          asm volatile("" : "+v"(r0));
+#pragma unroll
+          for (int fn = 0; fn < C::FN; ++fn) {
+            const int col = n0 + wn * C::TN + fn * 32 + (lane & 31);
+            const bool col_ok = !ragged || col < a.N;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+              const float v = acc[fm][fn][4 * q + rr];
+              if (v > tau4[rr] && col_ok) topk_push(S, r0 + rr, v, col);
+            }
           }
         }
         asm volatile("" ::: "memory");  // keep the threshold reads of later strips from being hoisted up here
@@ -417,7 +465,7 @@ __global__ void __launch_bounds__(C::NT) topk_kernel(TopkArgs a) {
         const int t = threadIdx.x;
         const int n = S.cnt[t];
         for (int i = 0; i < n; ++i) topk_insert(S.list_v[t], S.list_i[t], K, S.buf_v[t][i], S.buf_i[t][i]);
-        if (n) { S.tau[t] = S.list_v[t][K - 1]; S.cnt[t] = 0; }
+        settle(t, n != 0);
       }
     } else {
       // exact rescan: stage 8 columns of all 256 rows at a time, each row's owner inserts them
@@ -446,7 +494,7 @@ __global__ void __launch_bounds__(C::NT) topk_kernel(TopkArgs a) {
           }
         }
       }
-      if (threadIdx.x < C::BM) { S.tau[threadIdx.x] = S.list_v[threadIdx.x][K - 1]; S.cnt[threadIdx.x] = 0; }
+      if (threadIdx.x < C::BM) settle(threadIdx.x, true);
       if (threadIdx.x == 0) S.overflow = 0;
     }
     __syncthreads();
@@ -957,6 +1005,11 @@ __global__ void __launch_bounds__(256) generic_gemm_kernel(const half_t* __restr
 }
 
 // Plain copy, 16 bytes per thread step: the known-size kernel that HBM traffic counters are scaled by.
+__global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t* __restrict__ dst, uint32_t value, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = value;
+}
+
 __global__ void __launch_bounds__(256) copy_kernel(const uint4v* __restrict__ src, uint4v* __restrict__ dst, int64_t n16) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
@@ -1567,7 +1620,7 @@ size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K) {
   if (K > TOPK_MAX) return (size_t)B * (size_t)round_up(L, 8) * 2;  // the logits of every row
   int tm, tn, ng, grid;
   topk_plan(B, L, tm, tn, ng, grid);
-  return (size_t)ng * B * K * 8;
+  return (size_t)ng * B * K * 8 + (size_t)B * 4;  // the groups' candidate lists, the rows' shared bounds
 }
 
 int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, int64_t L, int64_t d, int64_t numy,
@@ -1600,13 +1653,17 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   TopkArgs a;
   int grid;
   topk_plan(B, L, a.tiles_m, a.tiles_n, a.n_groups, grid);
-  const size_t need = (size_t)a.n_groups * B * K * 8;
+  const size_t need = (size_t)a.n_groups * B * K * 8 + (size_t)B * 4;
   if (!workspace || workspace_bytes < need) return XFC_ERR_WORKSPACE;
   a.X = (const half_t*)X; a.ldx = ldx; a.W = (const half_t*)W; a.ldw = ldw;
   a.M = (int)B; a.N = (int)L; a.K = (int)d; a.topk = K;
   a.cand_v = reinterpret_cast<float*>(workspace);
   a.cand_i = reinterpret_cast<int32_t*>(a.cand_v + (size_t)a.n_groups * B * K);
+  a.bound = reinterpret_cast<uint32_t*>(a.cand_i + (size_t)a.n_groups * B * K);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  // a kernel, not a memset: the call may be recorded into a graph
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(B, 256)), dim3(256), 0, st, a.bound, 0u, B);
+  if (int rc0 = check_launch()) return rc0;
   const dim3 tg((unsigned)grid), tb(FwdCore::NT);
   int rc;
   switch (row_tile(B)) {
