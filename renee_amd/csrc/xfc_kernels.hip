@@ -174,7 +174,12 @@ __global__ void __launch_bounds__(C::NT) fwd_kernel(FwdArgs a) {
       for (int fn = 0; fn < C::FN; ++fn) words[fm][fn] = 0u;
     bool has_pos = false;
     if constexpr (MODE == FWD_GRAD) {
-      const int s = a.bucket_ptr[nt], e = a.bucket_ptr[nt + 1];
+      // read through the scalar path (the tile id is uniform and the table is read-only here): a vector
+      // load would make the compiler wait for every outstanding vector-memory operation before the first
+      // use, which includes the next tile's operand fetches that the main loop has just issued
+      typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+      const const_i32_ptr bp = (const_i32_ptr)(uintptr_t)a.bucket_ptr;
+      const int s = bp[nt], e = bp[nt + 1];
       has_pos = e > s;
       if (has_pos) {
         __syncthreads();  // every wave is done staging the previous tile
