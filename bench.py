@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
 # HBM bytes per launch of the dW+update kernel: rocprofv3 --pmc FETCH_SIZE (KiB, x2.000 from the 1 GiB
 # copy in the same run) + WRITE_SIZE (KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
-DW_UPDATE_TRAFFIC_BYTES = {2: (2 * 2834500.9 + 3932160.0) * 1024.0}
+DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2792275.6 + 1.000 * 3932160.0) * 1024.0}
 
 
 def _oracle_steps(B, L, d, c, seed, n_max, budget_s, warm):
