@@ -102,7 +102,7 @@ def cpu_baseline_cfg0(d: int, seed: int):
 
 
 def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: bool = True, scorers: bool = False,
-                batch: int = 0):
+                batch: int = 0, loss_variant: bool = False):
     """Times `steps` steps of one BASELINE configuration (with `batch` rows instead of its own when
     given), each from the same (W0, M1) state."""
     import torch
@@ -167,6 +167,20 @@ def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: boo
             step()
         torch.cuda.synchronize()
         out["drifting_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+    if loss_variant:
+        # the forward pass of the reference's one step in a hundred: the same kernel with the summed BCE loss
+        restore()
+        loss = torch.zeros(1, device=dev, dtype=torch.float32)
+        layer.fwd_grad(X, rowptr=rowptr, colidx=colidx, loss_out=loss)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = 5
+        e0.record()
+        for _ in range(n):
+            layer.fwd_grad(X, rowptr=rowptr, colidx=colidx, loss_out=loss)
+        e1.record()
+        torch.cuda.synchronize()
+        out["fwd_grad_with_loss_ms"] = e0.elapsed_time(e1) / n
     if scorers:
         restore()
         for K in (5, 100):
@@ -291,7 +305,7 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
     dev = torch.device("cuda:0")
-    r = time_config(args.config, args.steps, args.warmup, args.seed, dev)
+    r = time_config(args.config, args.steps, args.warmup, args.seed, dev, loss_variant=True)
     s = summarise(r)
     B, L, d = r["B"], r["L"], r["d"]
     gemm_flop = 2.0 * B * L * d
@@ -317,6 +331,7 @@ def main() -> int:
         "step_tflops": s["step_tflops"],
         "mfma_peak_frac": s["mfma_peak_frac"],
         "kernels_ms": s["kernels_ms"],
+        "fwd_grad_with_loss_ms": r.get("fwd_grad_with_loss_ms"),
         "kernels_tflops": {"fwd_grad": gemm_flop / k_ms[0] / 1e9, "dx": gemm_flop / k_ms[1] / 1e9,
                            "dw_update": gemm_flop / k_ms[2] / 1e9},
         "roofline": {"kernel": "dw_kernel<DW_UPDATE> (dW GEMM + SGD-momentum update)", "bound": "hbm",
