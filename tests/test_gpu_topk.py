@@ -76,6 +76,25 @@ def test_topk_exact_ties_and_pad_clamp(dev):
     assert int(i2.max()) <= 1989
 
 
+def test_topk_heavy_ties_across_label_groups(dev):
+    """Integer-valued scores: thousands of exact ties per row, spread over all the label groups that
+    share a row's score bound.  Ties with a published bound must still be admitted (a tying label of
+    lower id ranks first), so indices and values must equal a stable descending sort exactly; the
+    all-zero matrix is the extreme case (every score ties, and the bound is zero)."""
+    g = torch.Generator().manual_seed(11)
+    B, L, d = 70, 20011, 64
+    X = torch.randint(0, 2, (B, d), generator=g).half()
+    for W in (torch.randint(-1, 2, (L, d), generator=g).half(), torch.zeros(L, d).half()):
+        Z = X.float() @ W.float().T  # small integers, exact in fp16 products and fp32 sums
+        sv, si = torch.sort(Z, dim=1, descending=True, stable=True)
+        lay = XFCLayer(L, d, B, dev, weight=W)
+        for K in (1, 5, 8):
+            print(f"topk ties: B={B} L={L} K={K} zero={bool((W == 0).all())}", flush=True)
+            v, i = lay.topk(X.to(dev), K)
+            assert torch.equal(i.cpu(), si[:, :K])
+            assert torch.equal(v.cpu(), sv[:, :K])
+
+
 def test_topk_rising_scores_exact_rescan(dev):
     """Scores that keep rising with the label id beat every threshold in every tile: the per-row
     candidate buffers overflow and the exact rescan path must produce the answer."""
