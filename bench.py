@@ -37,7 +37,11 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
 # HBM bytes per launch of the dW+update kernel: rocprofv3 --pmc FETCH_SIZE (KiB, x2.000 from the 1 GiB
 # copy in the same run) + WRITE_SIZE (KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
-DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2792275.6 + 1.000 * 3932160.0) * 1024.0}
+DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2792275.6 + 1.000 * 3932160.0) * 1024.0,
+                           # the other configurations: profiles/xfc_step_other_configs_hbm_traffic_pmc.md
+                           1: (2.000 * 285086.0 + 1.000 * 393216.0) * 1024.0,
+                           3: (2.000 * 8560528.2 + 1.000 * 8436843.0) * 1024.0,
+                           4: (2.000 * 49418471.8 + 1.000 * 50331648.0) * 1024.0}
 
 
 def _oracle_steps(B, L, d, c, seed, n_max, budget_s, warm):
@@ -261,7 +265,7 @@ def master_weights_update(cfg: int, seed: int, dev):
             "hbm_frac": 18.0 * L * d / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
-def summarise(r):
+def summarise(r, cfg=None):
     """Per-configuration figures from time_config's result."""
     B, L, d = r["B"], r["L"], r["d"]
     gemm_flop = 2.0 * B * L * d
@@ -273,6 +277,9 @@ def summarise(r):
          "kernels_ms": {"fwd_grad(+bucket)": r["k_ms"][0], "dx(+reduce)": r["k_ms"][1], "dw_update": r["k_ms"][2]},
          "w_update_gbs": 8.0 * L * d / (r["k_ms"][2] * 1e-3) / 1e9,
          "w_update_hbm_frac": 8.0 * L * d / (r["k_ms"][2] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    if cfg in DW_UPDATE_TRAFFIC_BYTES:
+        s["dw_update_traffic"] = DW_UPDATE_TRAFFIC_BYTES[cfg]
+        s["dw_update_gbs_incl_measured_traffic"] = DW_UPDATE_TRAFFIC_BYTES[cfg] / (r["k_ms"][2] * 1e-3) / 1e9
     for k in ("drifting_ms_per_step", "top5_ms", "top100_ms"):
         if k in r:
             s[k] = r[k]
@@ -355,7 +362,7 @@ def main() -> int:
             if cfg == args.config:
                 continue
             others[f"configs[{cfg}]"] = summarise(time_config(cfg, n, 2, args.seed, dev, drifting=False,
-                                                              scorers=(cfg == 3)))
+                                                              scorers=(cfg == 3)), cfg)
             others[f"configs[{cfg}]"]["steps"] = n
         # what the 64-row tiles buy at batch 32: the same label count at batch 256 (one full-height tile)
         b256 = time_config(0, 20, 2, args.seed, dev, drifting=False, batch=256)["ms_per_step"]
