@@ -576,20 +576,27 @@ struct SelLds {
 // holds the K-th largest; when at most SEL_CAP elements lie in that bin or above, they are gathered and
 // sorted.  Otherwise pass 2 histograms the bin's low 5 bits to get the exact K-th key; elements above it
 // are gathered, and the elements equal to it are taken in label order until K are found.
+// With sample_stride > 1 the histogram is first taken over every sample_stride-th 16 KB block of the row
+// only: the K-th largest of a subset is never above the K-th largest of the row, so every element in that
+// bin or above is still a superset of the answer, about K * sample_stride elements; if they fit the sort
+// buffer the row has been read 1 + 1/sample_stride times instead of twice, and if not the full passes run.
 __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* __restrict__ logits, int64_t ldl, int L,
-                                                                   int64_t numy, int K, float* __restrict__ out_v,
+                                                                   int64_t numy, int K, int sample_stride,
+                                                                   float* __restrict__ out_v,
                                                                    int64_t* __restrict__ out_i) {
   __shared__ SelLds S;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint16_t* row = reinterpret_cast<const uint16_t*>(logits) + (int64_t)blockIdx.x * ldl;
-  auto for_each = [&](auto&& f) {
-    for (int i = tid * 8; i < L; i += SEL_THREADS * 8) {
+  auto for_each_block = [&](int block_stride, auto&& f) {
+    for (int64_t i64 = tid * 8; i64 < L; i64 += (int64_t)SEL_THREADS * 8 * block_stride) {
+      const int i = (int)i64;
       const uint4v q = *reinterpret_cast<const uint4v*>(row + i);
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         if (i + e < L) f(sel_key((q[e >> 1] >> (16 * (e & 1))) & 0xffffu), i + e);
     }
   };
+  auto for_each = [&](auto&& f) { for_each_block(1, f); };
   auto push = [&](uint32_t key, int idx) {
     const int slot = atomicAdd(&S.n_cand, 1);
     if (slot < SEL_CAP) S.cand[slot] = ((unsigned long long)(0xffffu - key) << 32) | (uint32_t)idx;
@@ -624,14 +631,37 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
   for (int b = tid; b < SEL_BINS; b += SEL_THREADS) S.hist[b] = 0;
   if (tid == 0) S.n_cand = 0;
   __syncthreads();
-  for_each([&](uint32_t key, int) { atomicAdd(&S.hist[key >> 5], 1); });
-  __syncthreads();
-  find_bin(SEL_BINS, 0);
-  __syncthreads();
-  const int bin = S.bin, above = S.above;
-  const int in_bin = S.hist[bin];
-  __syncthreads();
-  if (above + in_bin <= SEL_CAP) {
+  bool done = false;
+  if (sample_stride > 1) {
+    for_each_block(sample_stride, [&](uint32_t key, int) { atomicAdd(&S.hist[key >> 5], 1); });
+    __syncthreads();
+    find_bin(SEL_BINS, 0);  // the host only asks for a sample that holds at least K elements
+    __syncthreads();
+    const int sbin = S.bin;
+    for_each([&](uint32_t key, int idx) { if ((int)(key >> 5) >= sbin) push(key, idx); });
+    __syncthreads();
+    done = S.n_cand <= SEL_CAP;  // counts every push, also those that found the buffer full
+    __syncthreads();
+    if (!done) {
+      for (int b = tid; b < SEL_BINS; b += SEL_THREADS) S.hist[b] = 0;
+      if (tid == 0) S.n_cand = 0;
+      __syncthreads();
+    }
+  }
+  int bin = 0, above = 0, in_bin = 0;
+  if (!done) {
+    for_each([&](uint32_t key, int) { atomicAdd(&S.hist[key >> 5], 1); });
+    __syncthreads();
+    find_bin(SEL_BINS, 0);
+    __syncthreads();
+    bin = S.bin;
+    above = S.above;
+    in_bin = S.hist[bin];
+    __syncthreads();
+  }
+  if (done) {
+    // the sampled bound already gathered a superset of the answer
+  } else if (above + in_bin <= SEL_CAP) {
     for_each([&](uint32_t key, int idx) { if ((int)(key >> 5) >= bin) push(key, idx); });
   } else {
     if (tid < 64) S.hist[tid] = 0;
@@ -1648,8 +1678,14 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
       int rc = launch_fwd(FWD_LINEAR, (const half_t*)X + r0 * ldx, ldx, (const half_t*)W, ldw, (half_t*)workspace, ldl,
                           (int)rows, (int)L, (int)d, (int)L, 1.0f, 0.0f, nullptr, st);
       if (rc) return rc;
+      // sample every stride-th 16 KB block first when that still holds 16 K elements and points at about a
+      // thousand candidates at most (half the sort buffer)
+      int stride = 1;
+      while (stride < 16 && (int64_t)K * stride * 2 <= 1024 && L / (stride * 2) >= 16 * (int64_t)K &&
+             L / (stride * 2) >= (int64_t)SEL_THREADS * 8 * 4)
+        stride *= 2;
       hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)rows), dim3(SEL_THREADS), 0, st, (const half_t*)workspace,
-                         ldl, (int)L, numy, K, values + r0 * K, indices + r0 * K);
+                         ldl, (int)L, numy, K, stride, values + r0 * K, indices + r0 * K);
       rc = check_launch();
       if (rc) return rc;
     }

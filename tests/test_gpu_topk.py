@@ -195,6 +195,36 @@ def test_topk_select_crowded_bin_takes_the_refining_pass(dev):
     _check_select(dev, X, W, 128, vs_oracle=False)
 
 
+def test_topk_select_sampled_bound_and_its_fallback(dev):
+    """Rows long enough for the sampled first pass (every 8th 16 KB block at K = 100).  The sample's K-th
+    score only has to be a lower bound: rows whose large scores all sit in the sampled blocks, rows whose
+    sampled blocks hold only small scores (so that far more than the sort buffer lie above the bound and
+    the full passes must take over), and a crowd of equal top scores must all give the exact answer."""
+    g = torch.Generator().manual_seed(8)
+    L, K, blk = 300000, 100, 8192
+    in_sample = ((torch.arange(L) // blk) % 8 == 0)
+    base = (torch.rand(L, generator=g) * 0.5).half()
+    # (a) plain random scores
+    X, W = _axis_problem(base.clone())
+    _check_select(dev, X, W, K, vs_oracle=False)
+    # (b) everything large lies in the sampled blocks: the bound is tight, few candidates
+    s = base.clone()
+    s[in_sample] = (1.0 + torch.rand(int(in_sample.sum()), generator=g)).half()
+    X, W = _axis_problem(s)
+    _check_select(dev, X, W, K, vs_oracle=False)
+    # (c) the sampled blocks hold only small scores: the bound is loose and 200,000+ elements lie above it
+    s = base.clone()
+    s[~in_sample] = (1.0 + torch.rand(int((~in_sample).sum()), generator=g)).half()
+    X, W = _axis_problem(s)
+    _check_select(dev, X, W, K, vs_oracle=False)
+    # (d) 5000 copies of the largest score, spread everywhere
+    s = base.clone()
+    s[torch.randperm(L, generator=g)[:5000]] = 2.0
+    X, W = _axis_problem(s)
+    i = _check_select(dev, X, W, K, vs_oracle=False)
+    assert i[0].tolist() == sorted(i[0].tolist())  # equal scores come in label order
+
+
 def test_topk_select_many_copies_of_the_kth_value(dev):
     """3000 labels share the K-th largest score (more than can be sorted): they are taken in label order;
     also a constant row, signed zeros and negative scores."""
