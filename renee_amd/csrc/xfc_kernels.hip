@@ -1045,6 +1045,18 @@ __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t* __restrict__ ds
   if (i < n) dst[i] = value;
 }
 
+// bound[r] = key of a value safely below the K-th largest of row r's sample scores.  The sample scores
+// are fp16 roundings (half an ulp from the fp32 score at most), so one part in 1024 plus the smallest fp16
+// step below the K-th rounded score is below the K-th fp32 score of the sample, hence of the whole row.
+__global__ void __launch_bounds__(256) topk_seed_kernel(const float* __restrict__ sample_v, int K, uint32_t* __restrict__ bound,
+                                                        int64_t n) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= n) return;
+  const float x = sample_v[r * K + K - 1];
+  const float lo = x - (fabsf(x) * 0.0009765625f + 1.2e-7f);
+  bound[r] = (lo == lo && lo > -__builtin_huge_valf()) ? topk_key(lo) : 0u;  // NaN or -inf: no bound
+}
+
 __global__ void __launch_bounds__(256) copy_kernel(const uint4v* __restrict__ src, uint4v* __restrict__ dst, int64_t n16) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
@@ -1650,12 +1662,22 @@ static void topk_plan(int64_t B, int64_t L, int& tiles_m, int& tiles_n, int& n_g
   grid = tiles_m * n_groups;
 }
 
+// K <= 8: the rows' bounds start from the K-th score over a sample of the first TOPK_SAMPLE labels (a small
+// logits pass and an exact selection) when every label group has enough tiles for that to pay; otherwise
+// from nothing.  Without it every workgroup's first tiles overflow the candidate buffers and are rescanned.
+constexpr int TOPK_SAMPLE = 2048;
+static bool topk_seeded(int64_t L, int tiles_n, int n_groups) {
+  return L >= 8 * (int64_t)TOPK_SAMPLE && tiles_n >= 8 * n_groups;
+}
+
 size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K) {
   if (!dims_ok(B) || !dims_ok(L) || K < 1 || K > SEL_MAX_K || B == 0 || L == 0) return 0;
   if (K > TOPK_MAX) return (size_t)B * (size_t)round_up(L, 8) * 2;  // the logits of every row
   int tm, tn, ng, grid;
   topk_plan(B, L, tm, tn, ng, grid);
-  return (size_t)ng * B * K * 8 + (size_t)B * 4;  // the groups' candidate lists, the rows' shared bounds
+  size_t need = (size_t)ng * B * K * 8 + (size_t)round_up(B, 4) * 4;  // the groups' candidate lists, the rows' shared bounds
+  if (topk_seeded(L, tn, ng)) need += (size_t)B * TOPK_SAMPLE * 2 + (size_t)B * K * 12;  // sample logits, their top K
+  return need;
 }
 
 int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, int64_t L, int64_t d, int64_t numy,
@@ -1694,17 +1716,36 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   TopkArgs a;
   int grid;
   topk_plan(B, L, a.tiles_m, a.tiles_n, a.n_groups, grid);
-  const size_t need = (size_t)a.n_groups * B * K * 8 + (size_t)B * 4;
+  const bool seeded = topk_seeded(L, a.tiles_n, a.n_groups);
+  size_t need = (size_t)a.n_groups * B * K * 8 + (size_t)round_up(B, 4) * 4;
+  if (seeded) need += (size_t)B * TOPK_SAMPLE * 2 + (size_t)B * K * 12;
   if (!workspace || workspace_bytes < need) return XFC_ERR_WORKSPACE;
+  if (seeded && !aligned16(workspace)) return XFC_ERR_ALIGN;
   a.X = (const half_t*)X; a.ldx = ldx; a.W = (const half_t*)W; a.ldw = ldw;
   a.M = (int)B; a.N = (int)L; a.K = (int)d; a.topk = K;
   a.cand_v = reinterpret_cast<float*>(workspace);
   a.cand_i = reinterpret_cast<int32_t*>(a.cand_v + (size_t)a.n_groups * B * K);
   a.bound = reinterpret_cast<uint32_t*>(a.cand_i + (size_t)a.n_groups * B * K);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  // a kernel, not a memset: the call may be recorded into a graph
-  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(B, 256)), dim3(256), 0, st, a.bound, 0u, B);
-  if (int rc0 = check_launch()) return rc0;
+  if (seeded) {
+    // 16-byte aligned: the lists above are B * K * 8 * n_groups bytes (n_groups a multiple of 8), the bounds 16-byte padded
+    half_t* sample = reinterpret_cast<half_t*>(a.bound + round_up(B, 4));
+    int64_t* sample_i = reinterpret_cast<int64_t*>(sample + (size_t)B * TOPK_SAMPLE);
+    float* sample_v = reinterpret_cast<float*>(sample_i + (size_t)B * K);
+    int rc0 = launch_fwd(FWD_LINEAR, (const half_t*)X, ldx, (const half_t*)W, ldw, sample, TOPK_SAMPLE, (int)B, TOPK_SAMPLE,
+                         (int)d, TOPK_SAMPLE, 1.0f, 0.0f, nullptr, st);
+    if (rc0) return rc0;
+    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, (const half_t*)sample,
+                       (int64_t)TOPK_SAMPLE, TOPK_SAMPLE, (int64_t)TOPK_SAMPLE, K, 1, sample_v, sample_i);
+    if ((rc0 = check_launch())) return rc0;
+    hipLaunchKernelGGL(topk_seed_kernel, dim3((unsigned)ceil_div(B, 256)), dim3(256), 0, st, (const float*)sample_v, K,
+                       a.bound, B);
+    if ((rc0 = check_launch())) return rc0;
+  } else {
+    // a kernel, not a memset: the call may be recorded into a graph
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)ceil_div(B, 256)), dim3(256), 0, st, a.bound, 0u, B);
+    if (int rc0 = check_launch()) return rc0;
+  }
   const dim3 tg((unsigned)grid), tb(FwdCore::NT);
   int rc;
   switch (row_tile(B)) {

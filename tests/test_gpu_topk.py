@@ -95,6 +95,36 @@ def test_topk_heavy_ties_across_label_groups(dev):
             assert torch.equal(v.cpu(), sv[:, :K])
 
 
+def test_topk_bounds_seeded_from_the_label_sample(dev):
+    """Label counts large enough for the bounds to start from the K-th score over the first 2048 labels.
+    The seed only has to be a lower bound: rows whose best labels all lie inside the sample (the seed
+    then equals their K-th score up to the safety margin, and ties with it must survive), rows whose
+    sample holds nothing but their worst scores, and a sample of equal scores."""
+    g = torch.Generator().manual_seed(9)
+    L, K = 600000, 5
+    base = (torch.rand(L, generator=g) - 0.5).half()
+    cases = []
+    s = base.clone()
+    s[:2048] = (1.0 + torch.rand(2048, generator=g)).half()          # the best labels are the sampled ones
+    s[1000] = s[7] = s[2047] = s[:2048].max()                          # and the best score is shared
+    cases.append(s)
+    s = base.clone()
+    s[:2048] = -4.0                                                    # the sample is useless
+    s[599990] = s[300000] = 3.0
+    cases.append(s)
+    s = base.clone()
+    s[:2048] = 0.25                                                    # a flat sample inside the range
+    s[5000:5004] = 0.25                                                # later ties with the seed's score
+    cases.append(s)
+    for s in cases:
+        X, W = _axis_problem(s, B=2)                                   # rows: 1 x and 2 x the scores
+        lay = XFCLayer(L, 8, 2, dev, weight=W)
+        v, i = lay.topk(X.to(dev), K)
+        Z = X.float() @ W.float().T
+        sv, si = torch.sort(Z, dim=1, descending=True, stable=True)
+        assert torch.equal(i.cpu(), si[:, :K]) and torch.equal(v.cpu(), sv[:, :K])
+
+
 def test_topk_rising_scores_exact_rescan(dev):
     """Scores that keep rising with the label id beat every threshold in every tile: the per-row
     candidate buffers overflow and the exact rescan path must produce the answer."""
