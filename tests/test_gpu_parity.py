@@ -328,6 +328,28 @@ def test_state_dict_round_trip(dev):
     assert torch.equal(c.xfc_weight.cpu(), W) and float(c.momentum_buffer.abs().sum()) == 0.0
 
 
+def test_fp32_embeddings_are_cast_once_as_the_reference_casts_them(dev):
+    """The encoder hands over fp32 embeddings and the reference casts them to fp16 before the XFC GEMMs
+    (dl_base.py:561).  An fp32 `embed` (also one on the CPU) must give the bits the fp16 one gives, and
+    stay within tolerance of the oracle evaluated on the fp16-rounded embeddings."""
+    B, L, d = 96, 3000, 128
+    X32 = synth.make_X(B, d, 31)                      # fp32, not representable in fp16
+    W = synth.make_W(L, d, 31).half()
+    P = synth.make_positives(B, L, 8, 2.3, 1.1, 31)
+    px, py = P.coo()
+    a = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W)
+    b = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W)
+    c = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W)
+    dXa = a.xfc_backward(X32.to(dev), px, py).clone()           # fp32 on the GPU
+    dXb = b.xfc_backward(X32.half().to(dev), px, py).clone()    # already fp16
+    dXc = c.xfc_backward(X32, px, py).clone()                   # fp32 on the CPU
+    for other, dXo in ((b, dXb), (c, dXc)):
+        assert torch.equal(dXa, dXo) and torch.equal(a.xfc_weight, other.xfc_weight)
+        assert torch.equal(a.momentum_buffer, other.momentum_buffer)
+    ref = O.step(X32.half().float(), W.float(), torch.zeros(L, d), px, py, 0.05, 0.9, 0.0, 1.0)
+    assert rel(dXa[:B], ref["dX"]) <= TOL and rel(a.xfc_weight, ref["W"]) <= TOL
+
+
 def test_seeded_shape_sweep(dev):
     """Sixteen seeded shapes off every tile boundary (batch 1..520, labels 8..6000, d a multiple of 8 up
     to 384), X handed over as a strided view, random weight decay and loss scale: one whole step each."""
