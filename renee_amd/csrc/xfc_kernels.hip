@@ -209,6 +209,31 @@ __global__ void __launch_bounds__(C::NT) fwd_kernel(FwdArgs a) {
     auto body = [&](auto pos_tag, auto edge_tag) {
       constexpr bool POS = decltype(pos_tag)::value, EDGE = decltype(edge_tag)::value;
       float tile_loss = 0.f;
+      if constexpr (LOSS) {
+        static_assert(MODE == FWD_GRAD && !BETA, "the loss is that of the plain logits");
+        // The loss terms in a pass of their own over the accumulators, one block at a time: interleaved
+        // with the sigmoid and the staging below, the scheduler keeps dozens of elements in flight to
+        // hide the transcendentals' latency and spills hundreds of registers.
+        // softplus(z) = max(z,0) + log(1 + e^-|z|), minus z where the label is positive (dl_base.py:578-583)
+#pragma unroll
+        for (int fm = 0; fm < C::FM; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < C::FN; ++fn) {
+            const int ecol = n0 + wn * C::TN + fn * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float v = acc[fm][fn][r];
+              float t = fmaxf(v, 0.f) + 0.69314718f * __log2f(1.0f + __expf(-fabsf(v)));
+              if constexpr (POS) t -= v * (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
+              if constexpr (EDGE) {
+                const int erow = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
+                t = (erow < a.M && ecol < a.N) ? t : 0.f;
+              }
+              tile_loss += t;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+      }
 #pragma unroll
       for (int fm = 0; fm < C::FM; ++fm) {
 #pragma unroll
@@ -227,22 +252,11 @@ __global__ void __launch_bounds__(C::NT) fwd_kernel(FwdArgs a) {
               } else if constexpr (MODE == FWD_SIGMOID) {
                 v *= a.alpha;
               }
-              if constexpr (LOSS) {
-                // softplus(z) = max(z,0) + log(1 + e^-|z|), minus z where the label is positive (dl_base.py:578-583)
-                const int erow = m0 + wm * C::TM + fm * 32 + c_row(r, lane);
-                float t = fmaxf(v, 0.f) + 0.69314718f * __log2f(1.0f + __expf(-fabsf(v)));
-                if constexpr (POS) t -= v * (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
-                if constexpr (EDGE) t = (erow < a.M && ecol < a.N) ? t : 0.f;
-                tile_loss += t;
-              }
               if constexpr (MODE != FWD_LINEAR) v = sigmoidf_fast(v);
               if constexpr (POS) v -= (float)((words[fm][fn] >> c_row(r, lane)) & 1u);
               if constexpr (EDGE) { if (ecol >= a.N) v = 0.f; }
               stg[(4 * h + rr) * C::TN + fn * 32 + (lane & 31)] = (half_t)v;
             }
-            // with the loss terms the scheduler otherwise interleaves dozens of elements to hide the
-            // transcendental latency and spills hundreds of registers
-            if constexpr (LOSS) __builtin_amdgcn_sched_barrier(0);
           }
           // the wave's LDS traffic is ordered: its own writes above are visible to the reads below
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
