@@ -130,7 +130,11 @@ int xfc_fwd_grad_csr_static(const void* X, int64_t ldx, const void* W, int64_t l
  * dX[B x d] (fp32) = scale * G[B x L] . W[L x d].
  * Replaces dl_base.py:602-608 (torch.addmm with alpha = loss scale; the dead
  * split-K call at :604).  Needs ldg >= round_up(L,8) with zeroed pad columns
- * (xfc_fwd_grad_* writes them) and xfc_dx_workspace_bytes(B, L, d) of workspace.
+ * (xfc_fwd_grad_* writes them) and a workspace.  xfc_dx_workspace_bytes(B, L, d) is what the
+ * fastest split of the label axis needs (slices x B x d x 4 bytes); it is NOT monotone in B (a
+ * smaller batch may be cut into more slices), so size a buffer that serves several batch sizes
+ * with xfc_layer_workspace_bytes().  A smaller workspace is accepted down to 8 x B x d x 4 bytes:
+ * the label axis is then cut into as many slices as fit.
  */
 size_t xfc_dx_workspace_bytes(int64_t B, int64_t L, int64_t d);
 int xfc_dx(const void* G, int64_t ldg, const void* W, int64_t ldw, float* dX, int64_t lddx,
@@ -213,13 +217,25 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* M, int6
  *     rows are then processed in blocks of a multiple of 256.
  * Scores are expected to be finite: NaN and -inf are never selected by the K <= 8 pass, and a row with
  * fewer than K selectable scores reports (-inf, numy-1) in the remaining places.
- * Workspace: xfc_topk_workspace_bytes(B, L, K) bytes.
+ * Workspace: 16-byte aligned (for every K), xfc_topk_workspace_bytes(B, L, K) bytes.  For K <= 8 that is
+ * the need of the fastest plan (label groups x B x K x 8 bytes and small extras) and is NOT monotone in B (a
+ * smaller batch has fewer row tiles and so more label groups); a smaller workspace is accepted down to the
+ * need of 8 label groups.  Use xfc_layer_workspace_bytes() for a buffer that serves every batch size.
  */
 size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K);
 int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw,
              int64_t B, int64_t L, int64_t d, int64_t numy, int K,
              float* values, int64_t* indices,
              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * One workspace for every call of a layer: the largest need of xfc_step_csr (= xfc_fwd_grad_* + xfc_dx)
+ * and of xfc_topk with K <= 8 over all batch sizes 1..max_batch, with at most max_nnz label pairs per
+ * batch.  The per-call *_workspace_bytes() functions are not monotone in B, so sizing by max_batch alone
+ * does not cover the smaller batches (the last partial batch of an epoch, --accum micro-batches:
+ * dl_base.py:318-340 runs any batch up to xfc_batch_size on the buffers allocated at dl_base.py:175-187).
+ */
+size_t xfc_layer_workspace_bytes(int64_t max_batch, int64_t L, int64_t d, int64_t max_nnz);
 
 /*
  * Plain device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte aligned

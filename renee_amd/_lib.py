@@ -38,6 +38,7 @@ _SIGNATURES = {
     "xfc_step_csr": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64,
                             _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
     "xfc_topk_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "xfc_layer_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "xfc_topk": (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp, _sz, _vp]),
     "xfc_copy": (_int, [_vp, _vp, _i64, _vp]),
 }

@@ -1286,7 +1286,11 @@ int launch_fwd(int mode, const half_t* X, int64_t ldx, const half_t* W, int64_t 
 // count minimises a cost model fitted to measurements: workgroups run in rounds of one per CU, every
 // workgroup pays a fixed prologue + partial-tile store, and the partial sums are written and read once.
 // A stage of a smaller row tile takes proportionally less time.
-void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& k_per_split) {
+// With ws_limit the choice is restricted to slice counts whose partial sums fit that many bytes (8 slices, the
+// minimum, is always a candidate: the caller checks the final need).  The unrestricted need is not monotone in M
+// (a smaller batch may pick more slices), so a workspace sized for one batch serves smaller ones through this limit.
+void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& k_per_split,
+             size_t ws_limit = ~(size_t)0) {
   const int bm = row_tile(M);
   tiles_m = ceil_div(M, bm);
   tiles_n = ceil_div(N, DxCore::BN);
@@ -1299,6 +1303,7 @@ void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& 
   int best = 8;
   double best_cost = 0.0;
   for (int s = 8; s <= 256 && s <= max_s; s += 8) {
+    if (s > 8 && (size_t)s * (size_t)M * (size_t)N * 4 > ws_limit) break;
     const double rounds = (double)ceil_div(tiles * s, cus);
     const double cost = rounds * (nk / s + FIXED_STAGES) * STAGE_US + 2.0 * s * (double)M * N * 4.0 / PART_BYTES_PER_US;
     if (s == 8 || cost < best_cost) { best = s; best_cost = cost; }
@@ -1310,7 +1315,7 @@ void dx_plan(int M, int N, int K, int& tiles_m, int& tiles_n, int& splits, int& 
 int launch_dx(const half_t* G, int64_t ldg, const half_t* W, int64_t ldw, float* out, int64_t ldo, int M, int N, int K,
               float alpha, float beta, void* ws, size_t ws_bytes, hipStream_t st) {
   DxArgs a;
-  dx_plan(M, N, K, a.tiles_m, a.tiles_n, a.splits, a.k_per_split);
+  dx_plan(M, N, K, a.tiles_m, a.tiles_n, a.splits, a.k_per_split, ws ? ws_bytes : 0);
   const size_t need = (size_t)a.splits * M * N * 4;
   if (ws == nullptr || ws_bytes < need) return XFC_ERR_WORKSPACE;
   a.G = G; a.ldg = ldg; a.W = W; a.ldw = ldw; a.part = reinterpret_cast<float*>(ws);
@@ -1654,9 +1659,9 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int
                  const int32_t* colidx, int64_t nnz, void* G, int64_t ldg, float* dX, int64_t lddx, int64_t B,
                  int64_t L, int64_t d, float lr, float momentum, float weight_decay, float scale, void* workspace,
                  size_t workspace_bytes, void* stream) {
-  if (workspace_bytes < xfc_step_workspace_bytes(B, L, d, nnz) || !workspace) return XFC_ERR_WORKSPACE;
-  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
   const size_t off = (size_t)round_up(xfc_fwd_grad_workspace_bytes(L, nnz), 256);
+  if (!workspace || workspace_bytes < off) return XFC_ERR_WORKSPACE;  // xfc_dx checks its own share
+  if (ldg < round_up(L, 8)) return XFC_ERR_SHAPE;
   unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
   int rc = xfc_fwd_grad_csr(X, ldx, W, ldw, rowptr, colidx, G, ldg, B, L, d, nnz, nullptr, ws, off, stream);
   if (rc) return rc;
@@ -1665,7 +1670,25 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* Mo, int
   return xfc_dw_update(G, ldg, X, ldx, W, ldw, Mo, ldm, B, L, d, lr, momentum, weight_decay, nullptr, 0, stream);
 }
 
-static void topk_plan(int64_t B, int64_t L, int& tiles_m, int& tiles_n, int& n_groups, int& grid) {
+constexpr int TOPK_SAMPLE = 2048;
+// K <= 8: the rows' bounds start from the K-th score over a sample of the first TOPK_SAMPLE labels (a small
+// logits pass and an exact selection) when every label group has enough tiles for that to pay; otherwise
+// from nothing.  Without it every workgroup's first tiles overflow the candidate buffers and are rescanned.
+static bool topk_seeded(int64_t L, int tiles_n, int n_groups) {
+  return L >= 8 * (int64_t)TOPK_SAMPLE && tiles_n >= 8 * n_groups;
+}
+// bytes of the K <= 8 pass with n_groups label groups: the groups' candidate lists, the rows' shared bounds,
+// and (seeded) the sample logits and their top K
+static size_t topk_need(int64_t B, int64_t K, int n_groups, bool seeded) {
+  size_t need = (size_t)n_groups * B * K * 8 + (size_t)round_up(B, 4) * 4;
+  if (seeded) need += (size_t)B * TOPK_SAMPLE * 2 + (size_t)B * K * 12;
+  return need;
+}
+// Label groups of the K <= 8 pass: enough to give every CU a workgroup, fewer when the workspace holds no more
+// (8 at least; the seeding is dropped before the last groups are).  A smaller batch has fewer row tiles and so
+// more groups: the need is not monotone in B.
+static void topk_plan(int64_t B, int64_t L, int64_t K, size_t ws_limit, int& tiles_m, int& tiles_n, int& n_groups,
+                      int& grid, bool& seeded) {
   tiles_m = ceil_div(B, row_tile(B));
   tiles_n = ceil_div(L, FwdCore::BN);
   int per = num_cus() / (8 * tiles_m);  // groups per XCD
@@ -1673,25 +1696,36 @@ static void topk_plan(int64_t B, int64_t L, int& tiles_m, int& tiles_n, int& n_g
   n_groups = 8 * per;
   const int cap = (int)round_up(tiles_n, 8);
   if (n_groups > cap) n_groups = cap;
+  for (;; n_groups -= 8) {
+    seeded = topk_seeded(L, tiles_n, n_groups);
+    if (topk_need(B, K, n_groups, seeded) <= ws_limit) break;
+    if (seeded && topk_need(B, K, n_groups, false) <= ws_limit) { seeded = false; break; }
+    if (n_groups <= 8) break;  // the caller compares the need of this plan with what it was given
+  }
   grid = tiles_m * n_groups;
-}
-
-// K <= 8: the rows' bounds start from the K-th score over a sample of the first TOPK_SAMPLE labels (a small
-// logits pass and an exact selection) when every label group has enough tiles for that to pay; otherwise
-// from nothing.  Without it every workgroup's first tiles overflow the candidate buffers and are rescanned.
-constexpr int TOPK_SAMPLE = 2048;
-static bool topk_seeded(int64_t L, int tiles_n, int n_groups) {
-  return L >= 8 * (int64_t)TOPK_SAMPLE && tiles_n >= 8 * n_groups;
 }
 
 size_t xfc_topk_workspace_bytes(int64_t B, int64_t L, int64_t K) {
   if (!dims_ok(B) || !dims_ok(L) || K < 1 || K > SEL_MAX_K || B == 0 || L == 0) return 0;
   if (K > TOPK_MAX) return (size_t)B * (size_t)round_up(L, 8) * 2;  // the logits of every row
   int tm, tn, ng, grid;
-  topk_plan(B, L, tm, tn, ng, grid);
-  size_t need = (size_t)ng * B * K * 8 + (size_t)round_up(B, 4) * 4;  // the groups' candidate lists, the rows' shared bounds
-  if (topk_seeded(L, tn, ng)) need += (size_t)B * TOPK_SAMPLE * 2 + (size_t)B * K * 12;  // sample logits, their top K
-  return need;
+  bool seeded;
+  topk_plan(B, L, K, ~(size_t)0, tm, tn, ng, grid, seeded);
+  return topk_need(B, K, ng, seeded);
+}
+
+size_t xfc_layer_workspace_bytes(int64_t max_batch, int64_t L, int64_t d, int64_t max_nnz) {
+  if (!dims_ok(max_batch) || !dims_ok(L) || !dims_ok(d) || max_nnz < 0) return 0;
+  size_t dx = 0, topk = 0;
+  const int64_t k8 = L < TOPK_MAX ? L : TOPK_MAX;
+  for (int64_t b = 1; b <= max_batch; ++b) {
+    const size_t a = xfc_dx_workspace_bytes(b, L, d);
+    if (a > dx) dx = a;
+    const size_t t = k8 > 0 ? xfc_topk_workspace_bytes(b, L, k8) : 0;
+    if (t > topk) topk = t;
+  }
+  const size_t step = (size_t)round_up(xfc_fwd_grad_workspace_bytes(L, max_nnz), 256) + dx;
+  return step > topk ? step : topk;
 }
 
 int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, int64_t L, int64_t d, int64_t numy,
@@ -1729,12 +1763,11 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
   }
   TopkArgs a;
   int grid;
-  topk_plan(B, L, a.tiles_m, a.tiles_n, a.n_groups, grid);
-  const bool seeded = topk_seeded(L, a.tiles_n, a.n_groups);
-  size_t need = (size_t)a.n_groups * B * K * 8 + (size_t)round_up(B, 4) * 4;
-  if (seeded) need += (size_t)B * TOPK_SAMPLE * 2 + (size_t)B * K * 12;
+  bool seeded;
+  topk_plan(B, L, K, workspace ? workspace_bytes : 0, a.tiles_m, a.tiles_n, a.n_groups, grid, seeded);
+  const size_t need = topk_need(B, K, a.n_groups, seeded);
   if (!workspace || workspace_bytes < need) return XFC_ERR_WORKSPACE;
-  if (seeded && !aligned16(workspace)) return XFC_ERR_ALIGN;
+  if (!aligned16(workspace)) return XFC_ERR_ALIGN;
   a.X = (const half_t*)X; a.ldx = ldx; a.W = (const half_t*)W; a.ldw = ldw;
   a.M = (int)B; a.N = (int)L; a.K = (int)d; a.topk = K;
   a.cand_v = reinterpret_cast<float*>(workspace);

@@ -221,11 +221,12 @@ class XFCLayer:
         self.outsoft = torch.empty(self.max_batch, self.ldg, device=self.device, dtype=torch.float16)
         self.grad_input = torch.empty(self.max_batch, self.dims, device=self.device, dtype=torch.float32)
         self.xfc_weight_grad = None  # fp32 accumulator, only under split accumulation
+        self._g_live = False  # outsoft holds a G that dw_update / dw_accumulate has not consumed yet
         L = lib()
         with torch.cuda.device(self.device):
             check(L.xfc_init(), "xfc_init")
-            need = max(L.xfc_step_workspace_bytes(self.max_batch, self.numy, self.dims, self.max_positives),
-                       L.xfc_topk_workspace_bytes(self.max_batch, self.numy, min(8, self.numy)), 256)
+            # the largest need over every batch size up to max_batch: the per-call needs are not monotone in B
+            need = max(L.xfc_layer_workspace_bytes(self.max_batch, self.numy, self.dims, self.max_positives), 256)
             self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
 
     # -- helpers ---------------------------------------------------------------------------
@@ -280,16 +281,23 @@ class XFCLayer:
         check(rc, "xfc_logits")
         return out
 
-    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None):
+    def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None, overwrite_g: bool = False):
         """Exact top-K labels per row over all labels (FullPredictor's scoring loop, dl_base.py:736-756,
         with the pad clamp of :782 when numy < the stored label count).  Returns (values fp32, indices
         int64), each (batch, K); ties go to the lower label id.  K <= 1024: up to 8 in one fused pass,
         above that (the final evaluation's K = 100, dl_base.py:817-818) by an exact selection over the
-        fp16 logits, which are written to `outsoft` as the reference's scorer does (dl_base.py:745)."""
+        fp16 logits, which are written to `outsoft` as the reference's scorer does (dl_base.py:745).
+        K > 8 therefore destroys a G that fwd_grad left in `outsoft`: between fwd_grad and the dw_update /
+        dw_accumulate that consumes it the call raises unless overwrite_g=True."""
         x = self._x16(embed)
         bsz = x.shape[0]
         _require(1 <= K <= 1024 and K <= self.numy, "K must be in 1..min(1024, numy)")
         _require(bsz <= self.max_batch, "batch larger than max_batch")
+        _require(K <= 8 or overwrite_g or not self._g_live,
+                 "topk with K > 8 writes its logits over outsoft, which holds a G that dw_update / dw_accumulate "
+                 "has not consumed yet; finish the step first or pass overwrite_g=True")
+        if K > 8:
+            self._g_live = False
         vals = torch.empty(bsz, K, device=self.device, dtype=torch.float32)
         inds = torch.empty(bsz, K, device=self.device, dtype=torch.int64)
         L = lib()
@@ -341,6 +349,8 @@ class XFCLayer:
                                         G.data_ptr(), ldg, bsz, self.numy, self.dims, lp,
                                         ws.data_ptr(), ws.numel(), _stream(x))
         check(rc, "xfc_fwd_grad")
+        if out is None:
+            self._g_live = True
         return G[:, : self.numy]
 
     def dx(self, bsz: int, grad_input: torch.Tensor | None = None, scale: float = 1.0,
@@ -381,6 +391,7 @@ class XFCLayer:
                                                 self.lr if lr is None else float(lr), self.momentum, self.weight_decay,
                                                 None if dW_out is None else dW_out.data_ptr(), self.dims, _stream(x))
             check(rc, "xfc_dw_update_master")
+            self._g_live = self._g_live and out is not None
             return
         with torch.cuda.device(self.device):
             rc = lib().xfc_dw_update(G.data_ptr(), ldg, x.data_ptr(), x.stride(0),
@@ -389,6 +400,7 @@ class XFCLayer:
                                      self.weight_decay, None if dW_out is None else dW_out.data_ptr(), self.dims,
                                      _stream(x))
         check(rc, "xfc_dw_update")
+        self._g_live = self._g_live and out is not None
 
     def dw_accumulate(self, embed, out: torch.Tensor | None = None) -> None:
         """xfc_weight.grad (+)= G^T . embed for one micro-batch (dl_base.py:620-633)."""
@@ -402,6 +414,7 @@ class XFCLayer:
             rc = lib().xfc_dw(G.data_ptr(), G.stride(0), x.data_ptr(), x.stride(0), self.xfc_weight_grad.data_ptr(),
                               self.dims, bsz, self.numy, self.dims, 0.0 if first else 1.0, _stream(x))
         check(rc, "xfc_dw")
+        self._g_live = self._g_live and out is not None
 
     def optimizer_step(self, lr: float | None = None) -> None:
         """SGD-momentum on the accumulated fp32 grad, then drop it (dl_base.py:343-344)."""

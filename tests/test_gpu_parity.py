@@ -231,6 +231,88 @@ def test_xfc_gemm_three_modes(dev):
     assert rel(out2, torch.sigmoid(2.0 * O.logits(*ref) + 0.5 * prev.float())) <= TOL
 
 
+def test_xfc_gemm_alpha_beta_off_the_reference_call_sites(dev):
+    """Argument values the reference's three call sites never pass but its kernels accept
+    (xfc_gemm_kernel.cu:76-81, :137-142, :215-220 hand alpha and beta straight to the epilogue): beta != 0 in
+    the row x row mode, beta outside {0, 1} in the column x row mode and in xfc_dw, and an output whose
+    column stride is not 1 at a shape of many tiles."""
+    from renee_amd._lib import check, lib
+
+    B, L, d = 200, 4104, 72
+    g = torch.Generator().manual_seed(11)
+    G = (torch.rand(B, L, generator=g) - 0.3).half()
+    W = (torch.randn(L, d, generator=g) * 0.05).half()
+    X = torch.randn(B, d, generator=g).half()
+    Gd, Wd, Xd = G.to(dev), W.to(dev), X.to(dev)
+    # row x row (the dX mode), beta != 0: the split partial sums are reduced onto beta * out
+    prev = torch.randn(B, d, generator=g)
+    gi = prev.to(dev)
+    xfc_gemm(Gd, Wd, gi, 3.0, -0.5, False)
+    assert rel(gi, 3.0 * (G.float() @ W.float()) - 0.5 * prev) <= TOL
+    # column x row (the dW mode), alpha and beta arbitrary
+    prev = torch.randn(L, d, generator=g)
+    grad = prev.to(dev)
+    xfc_gemm(Gd.t(), Xd, grad, 2.0, -0.25, False)
+    assert rel(grad, 2.0 * (G.float().t() @ X.float()) - 0.25 * prev) <= TOL
+    # xfc_dw (split accumulation entry point) with a beta that is neither 0 nor 1
+    grad = prev.to(dev)
+    check(lib().xfc_dw(Gd.data_ptr(), Gd.stride(0), Xd.data_ptr(), Xd.stride(0), grad.data_ptr(), d, B, L, d, 0.5,
+                       torch.cuda.current_stream().cuda_stream), "xfc_dw")
+    assert rel(grad, G.float().t() @ X.float() + 0.5 * prev) <= TOL
+    # outputs with a column stride other than 1 (any-stride kernel), several hundred thousand elements
+    out_t = torch.full((L, B), float("nan"), device=dev, dtype=torch.float16)
+    xfc_gemm(Xd, Wd.t(), out_t.t(), 1.0, 0.0, True)  # out is (B, L) with strides (1, B)
+    assert rel(out_t.t(), torch.sigmoid(X.float() @ W.float().t())) <= TOL
+    wide = torch.zeros(L, 2 * d, device=dev)
+    xfc_gemm(Gd.t(), Xd, wide[:, ::2], 1.0, 0.0, False)  # column stride 2
+    assert rel(wide[:, ::2], G.float().t() @ X.float()) <= TOL
+    assert float(wide[:, 1::2].abs().max()) == 0.0
+    wide = torch.zeros(B, 2 * d, device=dev)
+    xfc_gemm(Gd, Wd, wide[:, ::2], 1.0, 0.0, False)
+    assert rel(wide[:, ::2], G.float() @ W.float()) <= TOL
+    assert float(wide[:, 1::2].abs().max()) == 0.0
+
+
+def test_dx_and_topk_accept_a_workspace_smaller_than_their_fastest_plan(dev):
+    """xfc_dx cuts the label axis into as many slices as the workspace holds (8 at least) and xfc_topk (K <= 8)
+    uses as many label groups as fit (8 at least): the result does not depend on it; below the minimum the
+    calls report XFC_ERR_WORKSPACE."""
+    from renee_amd._lib import check, lib
+
+    h = lib()
+    st = torch.cuda.current_stream().cuda_stream
+    B, L, d = 96, 40000, 64
+    g = torch.Generator().manual_seed(12)
+    G = (torch.rand(B, L, generator=g) - 0.3).half().to(dev)
+    W = (torch.randn(L, d, generator=g) * 0.05).half().to(dev)
+    want = G.float() @ W.float()
+    full = h.xfc_dx_workspace_bytes(B, L, d)
+    least = 8 * B * d * 4
+    assert full > least
+    for nbytes in (full, (full + least) // 2, least):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        dX = torch.full((B, d), float("nan"), device=dev)
+        check(h.xfc_dx(G.data_ptr(), L, W.data_ptr(), d, dX.data_ptr(), d, B, L, d, 1.0, ws.data_ptr(), nbytes, st), "xfc_dx")
+        assert rel(dX, want) <= TOL
+    ws = torch.empty(least, dtype=torch.uint8, device=dev)
+    assert h.xfc_dx(G.data_ptr(), L, W.data_ptr(), d, dX.data_ptr(), d, B, L, d, 1.0, ws.data_ptr(), least - 16, st) == 4
+    X = torch.randn(B, d, generator=g).half().to(dev)
+    Z = X.float() @ W.float().t()
+    sv, si = torch.sort(Z, dim=1, descending=True, stable=True)
+    full = h.xfc_topk_workspace_bytes(B, L, 5)
+    least = 8 * B * 5 * 8 + 4 * B
+    assert full > 2 * least
+    for nbytes in (full, full // 2, least):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        v = torch.empty(B, 5, device=dev)
+        i = torch.empty(B, 5, device=dev, dtype=torch.int64)
+        check(h.xfc_topk(X.data_ptr(), d, W.data_ptr(), d, B, L, d, L, 5, v.data_ptr(), i.data_ptr(), ws.data_ptr(), nbytes, st),
+              "xfc_topk")
+        assert torch.allclose(v, sv[:, :5], rtol=0, atol=2e-5 * float(sv.abs().max()))
+        assert float((i == si[:, :5]).float().mean()) > 0.99
+    assert h.xfc_topk(X.data_ptr(), d, W.data_ptr(), d, B, L, d, L, 5, v.data_ptr(), i.data_ptr(), ws.data_ptr(), least - 16, st) == 4
+
+
 def test_xfc_gemm_any_stride_fallback_and_errors(dev):
     B, L, d = 9, 37, 20  # nothing is a multiple of 8
     g = torch.Generator().manual_seed(0)
@@ -564,3 +646,27 @@ def test_reference_loss_module_interface(dev):
     ref = O.step(X.float(), Wo, Mo, z[0], z[1], 0.05, 0.9, 0.0, 4096.0)
     assert rel(lay.grad_input[:B], ref["dX"]) <= TOL
     assert rel(lay.xfc_weight, ref["W"]) <= TOL and rel(lay.momentum_buffer, ref["M"]) <= TOL
+
+
+def test_autograd_wrapper_sends_grad_input_into_the_encoder_graph(dev):
+    """loss.backward() through xfc_loss gives the encoder what the reference hands to embed.backward
+    (dl_base.py:360): scale * G . W with the weights before the update, and the step's update is applied."""
+    from renee_amd import xfc_loss
+
+    B, L, d = 96, 3000, 64
+    X, W, P = _problem(B, L, d, seed=21)
+    px, py = P.coo()
+    ref = O.step(X.float(), W.float(), torch.zeros(L, d), px, py, 0.05, 0.9, 0.0, 8.0)
+    lay = XFCLayer(L, d, B, dev, lr=0.05, momentum=0.9, weight=W)
+    enc = torch.nn.Linear(d, d, bias=False).to(dev)   # stands for the encoder
+    with torch.no_grad():
+        enc.weight.copy_(torch.eye(d))
+    inp = X.float().to(dev)
+    embed = enc(inp)
+    loss = xfc_loss(embed, lay, px, py, scale=8.0, compute_loss=True)
+    loss.backward()
+    assert rel(enc.weight.grad, ref["dX"].t() @ X.float()) <= TOL    # d loss / d enc.weight = dX^T . inp
+    assert rel(lay.xfc_weight, ref["W"]) <= TOL
+    want_loss = torch.nn.functional.binary_cross_entropy_with_logits(
+        O.logits(X.float(), W.float()), (ref["G"] < 0).float(), reduction="sum")
+    assert abs(float(loss) - float(want_loss)) <= 1e-4 * float(want_loss), (float(loss), float(want_loss))

@@ -317,3 +317,24 @@ def test_g_row_stride_is_skewed_off_powers_of_two():
         assert ld % 8 == 0 and ld >= (L + 7) // 8 * 8 and ld - L < 2048 + 8
         assert (ld * 2) % 4096 == 256
     assert g_row_stride(9) == 16 and g_row_stride(1000) == 1000
+
+
+def test_layer_workspace_covers_every_batch_size_up_to_max_batch():
+    """The per-call workspace needs are not monotone in the batch size (the dX split plan and the top-K label
+    groups both grow when the batch shrinks past a row-tile boundary); a layer serves any batch up to max_batch
+    on buffers allocated once (dl_base.py:175-187, :318-340), so its workspace must cover the largest need."""
+    h = lib()
+    saw_non_monotone = False
+    for L in (70001, 1310720):
+        for dims in (8, 16, 32, 64, 768):
+            for max_batch in (300, 384, 512, 1024):
+                nnz = 64 * max_batch
+                have = h.xfc_layer_workspace_bytes(max_batch, L, dims, nnz)
+                at_max = max(h.xfc_step_workspace_bytes(max_batch, L, dims, nnz), h.xfc_topk_workspace_bytes(max_batch, L, 8))
+                for b in range(1, max_batch + 1):
+                    need = max(h.xfc_step_workspace_bytes(b, L, dims, nnz), h.xfc_topk_workspace_bytes(b, L, 8))
+                    assert need <= have, (L, dims, max_batch, b, need, have)
+                    saw_non_monotone |= need > at_max
+    assert saw_non_monotone  # the case this function exists for does occur in the sweep
+    # K below 8 never needs more than K = 8
+    assert h.xfc_topk_workspace_bytes(256, 70001, 5) <= h.xfc_layer_workspace_bytes(300, 70001, 16, 64 * 300)
