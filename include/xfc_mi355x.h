@@ -205,11 +205,11 @@ int xfc_step_csr(const void* X, int64_t ldx, void* W, int64_t ldw, void* M, int6
  *   the lower label id.
  * Replaces FullPredictor's scoring loop, dl_base.py:736-756 (xfc_forward into outsoft,
  * then torch.max K times with the winners overwritten, or torch.topk for K > 5) and the
- * pad clamp at dl_base.py:782: indices >= numy are returned as numy-1.  1 <= K <= 1024, K <= L.
+ * pad clamp at dl_base.py:782: indices >= numy are returned as numy-1.  1 <= K <= 8192, K <= L.
  *   K <= 8 (the reference's per-epoch K = 5): one fused pass, the logits are never
  *     written; values are the fp32 accumulators (the reference returns fp16-rounded logits).
- *   8 < K <= 1024 (the reference's final evaluation, K = 100, dl_base.py:817-818; torch.topk at
- *     dl_base.py:756 takes any K): the fp16
+ *   8 < K <= 8192 (the reference's final evaluation, K = 100, dl_base.py:817-818; torch.topk at
+ *     dl_base.py:756 takes any K; above 1024 the selection sorts in a 128 KB LDS buffer, one row per CU): the fp16
  *     logits of a block of rows go to the workspace and an exact selection kernel picks each
  *     row's K largest; values are those fp16 logits widened to fp32, ties are between equal
  *     fp16 values.  xfc_topk_workspace_bytes() asks for all B rows at once (B*round_up(L,8)*2

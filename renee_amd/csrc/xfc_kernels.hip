@@ -563,13 +563,16 @@ __global__ void __launch_bounds__(64) topk_merge_kernel(const float* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------
-// top-K for 8 < K <= 1024: exact selection over rows of fp16 logits (one workgroup per row)
+// top-K for 8 < K <= 8192: exact selection over rows of fp16 logits (one workgroup per row)
 // ---------------------------------------------------------------------------------------------
-constexpr int SEL_MAX_K = 1024;  // one output thread per rank; at most half the sort capacity
+constexpr int SEL_MAX_K = 8192;  // at most half the capacity of the larger sort buffer
 constexpr int SEL_THREADS = 1024;
 constexpr int SEL_BINS = 2048;  // histogram over the top 11 bits of the 16-bit key
-constexpr int SEL_CAP = 2048;   // candidates that are sorted in LDS
-static_assert(SEL_MAX_K <= SEL_THREADS && 2 * SEL_MAX_K <= SEL_CAP, "ranks per row");
+// candidates that are sorted in LDS: 2048 for K <= 1024 (the reference's K = 100 lives here), 16384 (128 KB of
+// LDS, one row per CU at a time) for K up to SEL_MAX_K
+constexpr int SEL_CAP_SMALL = 2048, SEL_CAP_LARGE = 16384;
+constexpr int SEL_SMALL_MAX_K = SEL_CAP_SMALL / 2;
+static_assert(2 * SEL_MAX_K <= SEL_CAP_LARGE, "ranks per row");
 
 // fp16 bit pattern -> 16-bit key that orders like the value (-0 counts as +0).
 __device__ __forceinline__ uint32_t sel_key(uint32_t h) {
@@ -578,6 +581,7 @@ __device__ __forceinline__ uint32_t sel_key(uint32_t h) {
 }
 __device__ __forceinline__ uint32_t sel_unkey(uint32_t k) { return (k & 0x8000u) ? (k & 0x7fffu) : (~k & 0xffffu); }
 
+template <int SEL_CAP>
 struct SelLds {
   int hist[SEL_BINS];
   unsigned long long cand[SEL_CAP];
@@ -594,11 +598,13 @@ struct SelLds {
 // only: the K-th largest of a subset is never above the K-th largest of the row, so every element in that
 // bin or above is still a superset of the answer, about K * sample_stride elements; if they fit the sort
 // buffer the row has been read 1 + 1/sample_stride times instead of twice, and if not the full passes run.
+template <int SEL_CAP>
 __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* __restrict__ logits, int64_t ldl, int L,
                                                                    int64_t numy, int K, int sample_stride,
                                                                    float* __restrict__ out_v,
                                                                    int64_t* __restrict__ out_i) {
-  __shared__ SelLds S;
+  extern __shared__ __attribute__((aligned(16))) unsigned char sel_raw[];
+  SelLds<SEL_CAP>& S = *reinterpret_cast<SelLds<SEL_CAP>*>(sel_raw);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint16_t* row = reinterpret_cast<const uint16_t*>(logits) + (int64_t)blockIdx.x * ldl;
   auto for_each_block = [&](int block_stride, auto&& f) {
@@ -748,16 +754,16 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
       }
       __syncthreads();
     }
-  if (tid < K) {
-    const unsigned long long c = S.cand[tid];
+  for (int r = tid; r < K; r += SEL_THREADS) {
+    const unsigned long long c = S.cand[r];
     const uint32_t hbits = sel_unkey(0xffffu - (uint32_t)(c >> 32));
     const uint16_t h16 = (uint16_t)hbits;
     half_t h;
     __builtin_memcpy(&h, &h16, 2);
     int64_t idx = (int64_t)(uint32_t)c;
     if (idx >= numy) idx = numy - 1;
-    out_v[(int64_t)blockIdx.x * K + tid] = (float)h;
-    out_i[(int64_t)blockIdx.x * K + tid] = idx;
+    out_v[(int64_t)blockIdx.x * K + r] = (float)h;
+    out_i[(int64_t)blockIdx.x * K + r] = idx;
   }
 }
 
@@ -1362,6 +1368,23 @@ int launch_generic(const void* in1, int64_t as0, int64_t as1, const void* in2, i
   return check_launch();
 }
 
+struct SelArgs {
+  const half_t* logits; int64_t ldl; int L; int64_t numy; int K; int stride; float* out_v; int64_t* out_i;
+};
+template <int CAP>
+int launch_select(int rows, const SelArgs& a, hipStream_t st) {
+  constexpr int LDS = (int)sizeof(SelLds<CAP>);
+  static_assert(LDS <= 160 * 1024, "LDS budget");
+  const hipError_t e = raise_lds_limit<topk_select_kernel<CAP>>(LDS);
+  if (e != hipSuccess) {
+    fprintf(stderr, "xfc: cannot raise the dynamic LDS limit to %d bytes: %s\n", LDS, hipGetErrorString(e));
+    return XFC_ERR_HIP;
+  }
+  hipLaunchKernelGGL(topk_select_kernel<CAP>, dim3((unsigned)rows), dim3(SEL_THREADS), LDS, st, a.logits, a.ldl, a.L, a.numy,
+                     a.K, a.stride, a.out_v, a.out_i);
+  return check_launch();
+}
+
 bool dims_ok(int64_t v) { return v >= 0 && v <= 0x7fffffff; }
 
 }  // namespace
@@ -1403,6 +1426,8 @@ int xfc_init(void) {
   fwd_limits(std::type_identity<FwdCore>{}, std::type_identity<DxCore>{});
   fwd_limits(std::type_identity<FwdCore128>{}, std::type_identity<DxCore128>{});
   fwd_limits(std::type_identity<FwdCore64>{}, std::type_identity<DxCore64>{});
+  keep(raise_lds_limit<topk_select_kernel<SEL_CAP_SMALL>>((int)sizeof(SelLds<SEL_CAP_SMALL>)));
+  keep(raise_lds_limit<topk_select_kernel<SEL_CAP_LARGE>>((int)sizeof(SelLds<SEL_CAP_LARGE>)));
   keep(raise_lds_limit<dw_kernel<DW_UPDATE>>(DW_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_OUT>>(DW_LDS_BYTES));
   keep(raise_lds_limit<dw_kernel<DW_UPDATE_MASTER>>(DW_LDS_BYTES));
@@ -1750,13 +1775,13 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
       if (rc) return rc;
       // sample every stride-th 16 KB block first when that still holds 16 K elements and points at about a
       // thousand candidates at most (half the sort buffer)
+      const int cap = K <= SEL_SMALL_MAX_K ? SEL_CAP_SMALL : SEL_CAP_LARGE;
       int stride = 1;
-      while (stride < 16 && (int64_t)K * stride * 2 <= 1024 && L / (stride * 2) >= 16 * (int64_t)K &&
+      while (stride < 16 && (int64_t)K * stride * 2 <= cap / 2 && L / (stride * 2) >= 16 * (int64_t)K &&
              L / (stride * 2) >= (int64_t)SEL_THREADS * 8 * 4)
         stride *= 2;
-      hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)rows), dim3(SEL_THREADS), 0, st, (const half_t*)workspace,
-                         ldl, (int)L, numy, K, stride, values + r0 * K, indices + r0 * K);
-      rc = check_launch();
+      const SelArgs sa = {(const half_t*)workspace, ldl, (int)L, numy, K, stride, values + r0 * K, indices + r0 * K};
+      rc = K <= SEL_SMALL_MAX_K ? launch_select<SEL_CAP_SMALL>((int)rows, sa, st) : launch_select<SEL_CAP_LARGE>((int)rows, sa, st);
       if (rc) return rc;
     }
     return XFC_OK;
@@ -1782,9 +1807,8 @@ int xfc_topk(const void* X, int64_t ldx, const void* W, int64_t ldw, int64_t B, 
     int rc0 = launch_fwd(FWD_LINEAR, (const half_t*)X, ldx, (const half_t*)W, ldw, sample, TOPK_SAMPLE, (int)B, TOPK_SAMPLE,
                          (int)d, TOPK_SAMPLE, 1.0f, 0.0f, nullptr, st);
     if (rc0) return rc0;
-    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(SEL_THREADS), 0, st, (const half_t*)sample,
-                       (int64_t)TOPK_SAMPLE, TOPK_SAMPLE, (int64_t)TOPK_SAMPLE, K, 1, sample_v, sample_i);
-    if ((rc0 = check_launch())) return rc0;
+    const SelArgs sa = {(const half_t*)sample, (int64_t)TOPK_SAMPLE, TOPK_SAMPLE, (int64_t)TOPK_SAMPLE, K, 1, sample_v, sample_i};
+    if ((rc0 = launch_select<SEL_CAP_SMALL>((int)B, sa, st))) return rc0;
     hipLaunchKernelGGL(topk_seed_kernel, dim3((unsigned)ceil_div(B, 256)), dim3(256), 0, st, (const float*)sample_v, K,
                        a.bound, B);
     if ((rc0 = check_launch())) return rc0;

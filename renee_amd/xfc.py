@@ -284,14 +284,15 @@ class XFCLayer:
     def topk(self, embed: torch.Tensor, K: int = 5, numy: int | None = None, overwrite_g: bool = False):
         """Exact top-K labels per row over all labels (FullPredictor's scoring loop, dl_base.py:736-756,
         with the pad clamp of :782 when numy < the stored label count).  Returns (values fp32, indices
-        int64), each (batch, K); ties go to the lower label id.  K <= 1024: up to 8 in one fused pass,
-        above that (the final evaluation's K = 100, dl_base.py:817-818) by an exact selection over the
-        fp16 logits, which are written to `outsoft` as the reference's scorer does (dl_base.py:745).
+        int64), each (batch, K); ties go to the lower label id.  K <= 8192: up to 8 in one fused pass,
+        above that (the final evaluation's K = 100, dl_base.py:817-818; torch.topk at :756) by an exact
+        selection over the fp16 logits, which are written to `outsoft` as the reference's scorer does
+        (dl_base.py:745).
         K > 8 therefore destroys a G that fwd_grad left in `outsoft`: between fwd_grad and the dw_update /
         dw_accumulate that consumes it the call raises unless overwrite_g=True."""
         x = self._x16(embed)
         bsz = x.shape[0]
-        _require(1 <= K <= 1024 and K <= self.numy, "K must be in 1..min(1024, numy)")
+        _require(1 <= K <= 8192 and K <= self.numy, "K must be in 1..min(8192, numy)")
         _require(bsz <= self.max_batch, "batch larger than max_batch")
         _require(K <= 8 or overwrite_g or not self._g_live,
                  "topk with K > 8 writes its logits over outsoft, which holds a G that dw_update / dw_accumulate "

@@ -186,7 +186,9 @@ def _check_select(dev, X, W, K, numy=None, max_ws=None, vs_oracle=True):
 
 @pytest.mark.parametrize("B,L,d,K", [(37, 1000, 64, 100), (256, 4096, 768, 100), (64, 70001, 128, 9),
                                      (5, 128, 8, 128), (3, 100, 8, 100), (9, 5000, 64, 500), (4, 1024, 8, 1024),
-                                     (6, 30000, 32, 1024)])
+                                     (6, 30000, 32, 1024),
+                                     # above 1024 the selection runs on its larger sort buffer (up to 8192)
+                                     (5, 9000, 32, 1025), (3, 8192, 8, 8192), (4, 200003, 64, 5000), (2, 70001, 16, 8192)])
 def test_topk_select_matches_sort_and_oracle(dev, B, L, d, K):
     X = synth.make_X(B, d, 4).half()
     W = synth.make_W(L, d, 4).half()
@@ -276,3 +278,16 @@ def test_topk_select_many_copies_of_the_kth_value(dev):
     Wz[::2, 0] = -0.0
     iz = _check_select(dev, Xz, Wz, 100, vs_oracle=False)
     assert iz[0].tolist() == list(range(100)) and iz[1].tolist() == list(range(100))
+
+
+def test_topk_select_large_k_with_heavy_ties(dev):
+    """K above 1024 on rows that hold few distinct scores: the K-th value's copies outnumber the sort buffer and
+    are taken in label order; the result is still the stable sort's."""
+    B, L, d = 3, 60000, 8
+    g = torch.Generator().manual_seed(9)
+    X = torch.zeros(B, d)
+    X[:, 0] = 1.0
+    W = torch.zeros(L, d)
+    W[:, 0] = torch.randint(0, 3, (L,), generator=g).float() * 0.25     # three distinct scores, ~20,000 copies each
+    _check_select(dev, X.half(), W.half(), 6000, vs_oracle=False)
+    _check_select(dev, X.half(), W.half(), 1500, vs_oracle=False)

@@ -175,7 +175,7 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
                    'int main(void) {\n'
                    '  if (xfc_abi_version() != XFC_ABI_VERSION) return 1;\n'
                    '  if (xfc_logits(NULL, 8, NULL, 8, NULL, 8, 4, 4, 8, NULL) != XFC_ERR_INVALID) return 2;\n'
-                   '  if (xfc_topk_workspace_bytes(4, 1000, 1025) != 0) return 3;\n'
+                   '  if (xfc_topk_workspace_bytes(4, 10000, 8193) != 0) return 3;\n'
                    '  if (xfc_topk_workspace_bytes(4, 1000, 100) != (size_t)4 * 1000 * 2) return 4;\n'
                    '  printf("%s\\n", xfc_strerror(XFC_ERR_WORKSPACE));\n  return 0;\n}\n')
     exe = tmp_path / "t"
