@@ -106,7 +106,7 @@ def cpu_baseline_cfg0(d: int, seed: int):
             "s_per_step_median": t, "s_per_step_min": ts[0], "gflops": 6.0 * B * L * d / t / 1e9}
 
 
-def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: bool = True, scorers: bool = False,
+def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, wall_clock: bool = True, scorers: bool = False,
                 batch: int = 0, loss_variant: bool = False):
     """Times `steps` steps of one BASELINE configuration (with `batch` rows instead of its own when
     given), each from the same (W0, M1) state."""
@@ -166,7 +166,7 @@ def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, drifting: boo
     out = {"B": B, "L": L, "d": d, "nnz": P.nnz, "zipf": c["zipf"], "ms_per_step": ms_events, "k_ms": k_ms,
            "ms_events": {"mean": ms_events, "median": per_step[steps // 2], "min": per_step[0]},
            "wall_s_incl_restore": wall_with_restore}
-    if drifting:
+    if wall_clock:
         # the contract's figure: K steps back to back between two synchronisations, nothing else in between
         restore()
         torch.cuda.synchronize()
@@ -392,11 +392,11 @@ def main() -> int:
         for cfg, n in ((0, 20), (1, 20), (3, 6), (4, 3)):
             if cfg == args.config:
                 continue
-            others[f"configs[{cfg}]"] = summarise(time_config(cfg, n, 2, args.seed, dev, drifting=False,
+            others[f"configs[{cfg}]"] = summarise(time_config(cfg, n, 2, args.seed, dev, wall_clock=False,
                                                               scorers=(cfg == 3)), cfg)
             others[f"configs[{cfg}]"]["steps"] = n
         # what the 64-row tiles buy at batch 32: the same label count at batch 256 (one full-height tile)
-        b256 = time_config(0, 20, 2, args.seed, dev, drifting=False, batch=256)["ms_per_step"]
+        b256 = time_config(0, 20, 2, args.seed, dev, wall_clock=False, batch=256)["ms_per_step"]
         others["configs[0]"]["batch256_same_labels_ms_per_step"] = b256
         others["configs[0]"]["vs_quarter_of_batch256"] = others["configs[0]"]["ms_per_step"] / (b256 / 4.0)
         out["other_configs"] = others

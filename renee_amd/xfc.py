@@ -108,14 +108,19 @@ def read_sparse_labels(path: str):
 
     with open(path) as f:
         rows, cols = (int(v) for v in f.readline().split()[:2])
-        rowptr = np.zeros(rows + 1, dtype=np.int64)
-        colidx = []
-        for r in range(rows):
-            toks = f.readline().split()
-            ids = sorted({int(t.split(":")[0]) for t in toks})
-            colidx.extend(ids)
-            rowptr[r + 1] = rowptr[r] + len(ids)
-    return rowptr, np.asarray(colidx, dtype=np.int32), (rows, cols)
+        lines = f.read().split("\n")[:rows]
+    lines += [""] * (rows - len(lines))
+    # one pass of numpy over the whole text instead of a Python loop over tokens
+    counts = np.fromiter((ln.count(":") for ln in lines), dtype=np.int64, count=rows)
+    flat = np.array(" ".join(lines).replace(":", " ").split(), dtype=np.float64)
+    ids = flat[0::2].astype(np.int64)
+    _require(ids.shape[0] == int(counts.sum()), "malformed label file: expected col:val pairs")
+    row_of = np.repeat(np.arange(rows, dtype=np.int64), counts)
+    key = np.unique(row_of * max(cols, 1) + ids)          # sorted by (row, label), duplicates dropped
+    row_of, ids = key // max(cols, 1), key % max(cols, 1)
+    rowptr = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(np.bincount(row_of, minlength=rows), out=rowptr[1:])
+    return rowptr, ids.astype(np.int32), (rows, cols)
 
 
 def batch_positives(rowptr, colidx, ids, start_label: int = 0, end_label: int | None = None, device=None):

@@ -669,4 +669,5 @@ def test_autograd_wrapper_sends_grad_input_into_the_encoder_graph(dev):
     assert rel(lay.xfc_weight, ref["W"]) <= TOL
     want_loss = torch.nn.functional.binary_cross_entropy_with_logits(
         O.logits(X.float(), W.float()), (ref["G"] < 0).float(), reduction="sum")
-    assert abs(float(loss) - float(want_loss)) <= 1e-4 * float(want_loss), (float(loss), float(want_loss))
+    got_loss = float(loss.detach())
+    assert abs(got_loss - float(want_loss)) <= 1e-4 * float(want_loss), (got_loss, float(want_loss))
