@@ -25,6 +25,13 @@ def rel(a, b):
     return float((a - b).norm() / b.norm())
 
 
+def worst(a, b):
+    """Largest single error as a fraction of the largest reference magnitude.  The Frobenius norm hides a few
+    wrong rows or columns in a large matrix (seven wrong label rows of 3001 stay under 1e-3); this does not."""
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
 def _problem(B, L, d, kmax=8, kmean=2.3, zipf=1.1, seed=0):
     X = synth.make_X(B, d, seed).half()
     W = synth.make_W(L, d, seed).half()
@@ -46,6 +53,7 @@ def _check_step(dev, X, W, px, py, lr=0.05, mu=0.9, wd=0.0, scale=1.0, steps=1, 
         else:
             G = lay.fwd_grad(Xd, px.to(dev), py.to(dev))
         assert rel(G, ref["G"]) <= TOL
+        assert float((G.float().cpu() - ref["G"]).abs().max()) <= 1e-3   # |G| < 1: half an fp16 step is 2.4e-4
         if L % 8:  # the pad columns up to the next multiple of 8 are written as zero
             assert float(lay.outsoft[:B, L:(L + 7) // 8 * 8].abs().max()) == 0.0
         # every positive is negative in G, everything else is in (0, 1)
@@ -56,14 +64,14 @@ def _check_step(dev, X, W, px, py, lr=0.05, mu=0.9, wd=0.0, scale=1.0, steps=1, 
             mask[px[ok], py[ok]] = True
         assert (Gc[mask] <= 0).all() and (Gc[~mask] >= 0).all()
         dX = lay.dx(B, scale=scale)
-        assert rel(dX, ref["dX"]) <= TOL
+        assert rel(dX, ref["dX"]) <= TOL and worst(dX, ref["dX"]) <= 5e-3
         dW = torch.empty(L, d, device=dev, dtype=torch.float32)
         lay.dw_update(Xd, dW_out=dW)
-        assert rel(dW, ref["dW"]) <= TOL
+        assert rel(dW, ref["dW"]) <= TOL and worst(dW, ref["dW"]) <= 5e-3
         # update parity is judged from the same starting point: the oracle is advanced from the
         # device's fp16 state so that per-step rounding does not compound in the comparison
-        assert rel(lay.xfc_weight, ref["W"]) <= TOL
-        assert rel(lay.momentum_buffer, ref["M"]) <= TOL
+        assert rel(lay.xfc_weight, ref["W"]) <= TOL and worst(lay.xfc_weight, ref["W"]) <= 3e-3
+        assert rel(lay.momentum_buffer, ref["M"]) <= TOL and worst(lay.momentum_buffer, ref["M"]) <= 3e-3
         Wo, Mo = lay.xfc_weight.float().cpu(), lay.momentum_buffer.float().cpu()
     return lay
 
