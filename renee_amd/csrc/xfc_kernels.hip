@@ -43,19 +43,27 @@ __device__ __forceinline__ void xcd_map(int id, int n_inner, int& inner, int& ou
 // Output: bucket_ptr[n_tiles+1] and (ent_row, ent_col)[nnz] grouped by col / tile_w.
 // Pairs whose row or column is out of range are dropped.  The per-tile counters live in LDS when
 // they fit (IN_LDS, n_tiles <= BUCKET_LDS_TILES) and in the global scratch array `cursor` otherwise.
+// Both inputs are walked by entry, one coalesced load per thread and pass: a CSR entry finds its row by a
+// binary search of the row pointers, which are staged in LDS when they fit (ROWS_IN_LDS; otherwise the rows are
+// walked one per thread, each thread reading its row's labels one after the other -- as many dependent round
+// trips as the longest row has labels, which made this pass 17 us of a 4 ms step).
 constexpr int BUCKET_LDS_TILES = 12288;
+constexpr int BUCKET_DYN_LDS_MAX = 56 * 1024;  // next to the 4 KB of scan scratch, within the default 64 KB
 
-template <bool IN_LDS>
+template <bool IN_LDS, bool ROWS_IN_LDS>
 __global__ void __launch_bounds__(1024) bucket_positives_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ colidx, const int64_t* __restrict__ pos_x,
     const int64_t* __restrict__ pos_y, int64_t nnz, int B, int64_t L, int tile_w, int n_tiles,
     int32_t* __restrict__ bucket_ptr, int32_t* __restrict__ cursor_g, int32_t* __restrict__ ent_row,
     int32_t* __restrict__ ent_col) {
-  __shared__ int32_t part[1024];
-  extern __shared__ int32_t cursor_l[];
-  int32_t* cursor = IN_LDS ? cursor_l : cursor_g;
-  const int t = threadIdx.x;
+  __shared__ int32_t wave_tot[16];
+  extern __shared__ int32_t dyn_l[];
+  int32_t* cursor = IN_LDS ? dyn_l : cursor_g;
+  int32_t* rows_l = dyn_l + (IN_LDS ? n_tiles : 0);  // ROWS_IN_LDS: rowptr[0..B]
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   for (int i = t; i < n_tiles; i += 1024) cursor[i] = 0;
+  if constexpr (ROWS_IN_LDS)
+    for (int i = t; i <= B; i += 1024) rows_l[i] = rowptr[i];
   __syncthreads();
   // pass 0 counts, pass 1 places
   auto walk = [&](auto visit) {
@@ -63,6 +71,19 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
       for (int64_t p = t; p < nnz; p += 1024) {
         const int64_t r = pos_x[p], c = pos_y[p];
         if (r >= 0 && r < B && c >= 0 && c < L) visit((int)r, (int)c);
+      }
+    } else if constexpr (ROWS_IN_LDS) {
+      const int p0 = rows_l[0];
+      int64_t p1 = rows_l[B];
+      if (p1 > p0 + nnz) p1 = p0 + nnz;  // never past what the caller sized the entry arrays for
+      for (int64_t p = p0 + t; p < p1; p += 1024) {
+        const int64_t c = colidx[p];
+        int lo = 0, hi = B;  // the row b with rowptr[b] <= p < rowptr[b + 1]: first b whose rowptr[b + 1] > p
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (rows_l[mid + 1] > p) hi = mid; else lo = mid + 1;
+        }
+        if (lo < B && c >= 0 && c < L) visit(lo, (int)c);
       }
     } else {
       for (int b = t; b < B; b += 1024)
@@ -74,26 +95,35 @@ __global__ void __launch_bounds__(1024) bucket_positives_kernel(
   };
   walk([&](int, int c) { atomicAdd(&cursor[c / tile_w], 1); });
   __syncthreads();
+  // exclusive scan of the per-tile counts: each thread owns `per` consecutive tiles; lanes scan by shuffles,
+  // the sixteen waves' totals go through LDS
   const int per = (n_tiles + 1023) / 1024;
   const int lo = t * per, hi = min(n_tiles, lo + per);
   int s = 0;
   for (int i = lo; i < hi; ++i) s += cursor[i];
-  part[t] = s;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    const int v = t >= off ? part[t - off] : 0;
-    __syncthreads();
-    part[t] += v;
-    __syncthreads();
+  int inc = s;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int v = __shfl_up(inc, off, 64);
+    if (lane >= off) inc += v;
   }
-  int run = part[t] - s;
+  if (lane == 63) wave_tot[wave] = inc;
+  __syncthreads();
+  int before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const int v = wave_tot[w];
+    if (w < wave) before += v;
+    total += v;
+  }
+  int run = before + inc - s;
   for (int i = lo; i < hi; ++i) {
     const int c = cursor[i];
     bucket_ptr[i] = run;
     cursor[i] = run;
     run += c;
   }
-  if (t == 1023) bucket_ptr[n_tiles] = part[1023];
+  if (t == 1023) bucket_ptr[n_tiles] = total;
   __syncthreads();
   walk([&](int r, int c) {
     const int at = atomicAdd(&cursor[c / tile_w], 1);
@@ -1529,14 +1559,19 @@ static int fwd_grad_impl(const void* X, int64_t ldx, const void* W, int64_t ldw,
   BucketWs bk = carve_bucket_ws(ws, L, nnz);
   const int n_tiles = (int)round_up(ceil_div(L, FwdCore::BN), 8);
   const bool coo = pos_x != nullptr;
-  if (n_tiles <= BUCKET_LDS_TILES)
-    hipLaunchKernelGGL(bucket_positives_kernel<true>, dim3(1), dim3(1024), n_tiles * 4, st, coo ? nullptr : rowptr,
-                       coo ? nullptr : colidx, coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L,
-                       FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
-  else
-    hipLaunchKernelGGL(bucket_positives_kernel<false>, dim3(1), dim3(1024), 0, st, coo ? nullptr : rowptr,
-                       coo ? nullptr : colidx, coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L,
-                       FwdCore::BN, n_tiles, bk.bucket_ptr, bk.cursor, bk.ent_row, bk.ent_col);
+  const bool in_lds = n_tiles <= BUCKET_LDS_TILES;
+  const size_t dyn_tiles = in_lds ? (size_t)n_tiles * 4 : 0;
+  const bool rows_in_lds = !coo && dyn_tiles + ((size_t)B + 1) * 4 <= (size_t)BUCKET_DYN_LDS_MAX;
+  const size_t dyn = dyn_tiles + (rows_in_lds ? ((size_t)B + 1) * 4 : 0);
+  auto launch_bucket = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(1024), dyn, st, coo ? nullptr : rowptr, coo ? nullptr : colidx,
+                       coo ? pos_x : nullptr, coo ? pos_y : nullptr, nnz, (int)B, L, FwdCore::BN, n_tiles, bk.bucket_ptr,
+                       bk.cursor, bk.ent_row, bk.ent_col);
+  };
+  if (in_lds && rows_in_lds) launch_bucket(bucket_positives_kernel<true, true>);
+  else if (in_lds) launch_bucket(bucket_positives_kernel<true, false>);
+  else if (rows_in_lds) launch_bucket(bucket_positives_kernel<false, true>);
+  else launch_bucket(bucket_positives_kernel<false, false>);
   int rc = check_launch();
   if (rc) return rc;
   // label columns L .. round_up(L, 8) are written as zero so that G can be read in 16-byte
