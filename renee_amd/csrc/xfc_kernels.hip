@@ -1063,30 +1063,66 @@ __global__ void __launch_bounds__(DwCore::NT) dw_kernel(DwArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// any-stride fallback: one thread per output element
+// any-stride fallback: 64 x 64 output tile per workgroup, 4 x 4 outputs per thread, operands staged through LDS
+// as fp32 in 32-deep slabs.  Each output is one fp32 accumulator summed over k in ascending order.  A slab is
+// read with consecutive threads along whichever of its two axes has the smaller stride.
 // ---------------------------------------------------------------------------------------------
+constexpr int GEN_T = 64, GEN_K = 32, GEN_PAD = 4;
 __global__ void __launch_bounds__(256) generic_gemm_kernel(const half_t* __restrict__ A, int64_t as0, int64_t as1,
                                                            const half_t* __restrict__ Bm, int64_t bs0, int64_t bs1,
                                                            void* out, int64_t os0, int64_t os1, int M, int N, int K,
                                                            float alpha, float beta, int sigmoid, int out_half) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (int64_t)M * N) return;
-  const int m = (int)(idx / N), n = (int)(idx % N);
-  float s = 0.f;
-  for (int k = 0; k < K; ++k) s += (float)A[m * as0 + k * as1] * (float)Bm[k * bs0 + n * bs1];
-  s *= alpha;
-  const int64_t o = m * os0 + n * os1;
-  if (out_half) {
-    half_t* p = reinterpret_cast<half_t*>(out) + o;
-    if (beta != 0.f) s += beta * (float)*p;
-    if (sigmoid) s = sigmoidf_fast(s);
-    *p = (half_t)s;
-  } else {
-    float* p = reinterpret_cast<float*>(out) + o;
-    if (beta != 0.f) s += beta * *p;
-    if (sigmoid) s = sigmoidf_fast(s);
-    *p = s;
+  __shared__ __align__(16) float As[GEN_K][GEN_T + GEN_PAD];
+  __shared__ __align__(16) float Bs[GEN_K][GEN_T + GEN_PAD];
+  const int tiles_n = (N + GEN_T - 1) / GEN_T;
+  const int m0 = (int)(blockIdx.x / tiles_n) * GEN_T, n0 = (int)(blockIdx.x % tiles_n) * GEN_T;
+  const int t = threadIdx.x, ty = t >> 4, tx = t & 15;
+  const bool a_k_fast = (as1 < 0 ? -as1 : as1) <= (as0 < 0 ? -as0 : as0);
+  const bool b_k_fast = (bs0 < 0 ? -bs0 : bs0) <= (bs1 < 0 ? -bs1 : bs1);
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += GEN_K) {
+#pragma unroll
+    for (int j = 0; j < GEN_T * GEN_K / 256; ++j) {
+      const int i = t + j * 256;
+      int kk = a_k_fast ? i % GEN_K : i / GEN_T, mm = a_k_fast ? i / GEN_K : i % GEN_T;
+      As[kk][mm] = (m0 + mm < M && k0 + kk < K) ? (float)A[(int64_t)(m0 + mm) * as0 + (int64_t)(k0 + kk) * as1] : 0.f;
+      kk = b_k_fast ? i % GEN_K : i / GEN_T;
+      const int nn = b_k_fast ? i / GEN_K : i % GEN_T;
+      Bs[kk][nn] = (n0 + nn < N && k0 + kk < K) ? (float)Bm[(int64_t)(k0 + kk) * bs0 + (int64_t)(n0 + nn) * bs1] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GEN_K; ++kk) {
+      const float4 av = *reinterpret_cast<const float4*>(&As[kk][ty * 4]);
+      const float4 bv = *reinterpret_cast<const float4*>(&Bs[kk][tx * 4]);
+      const float a4[4] = {av.x, av.y, av.z, av.w}, b4[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += a4[i] * b4[j];
+    }
+    __syncthreads();
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+      if (m >= M || n >= N) continue;
+      float v = acc[i][j] * alpha;
+      const int64_t o = (int64_t)m * os0 + (int64_t)n * os1;
+      if (out_half) {
+        half_t* p = reinterpret_cast<half_t*>(out) + o;
+        if (beta != 0.f) v += beta * (float)*p;
+        if (sigmoid) v = sigmoidf_fast(v);
+        *p = (half_t)v;
+      } else {
+        float* p = reinterpret_cast<float*>(out) + o;
+        if (beta != 0.f) v += beta * *p;
+        if (sigmoid) v = sigmoidf_fast(v);
+        *p = v;
+      }
+    }
 }
 
 // Plain copy, 16 bytes per thread step: the known-size kernel that HBM traffic counters are scaled by.
@@ -1390,9 +1426,10 @@ int launch_dw(int mode, DwArgs a, hipStream_t st) {
 int launch_generic(const void* in1, int64_t as0, int64_t as1, const void* in2, int64_t bs0, int64_t bs1, void* out,
                    int64_t os0, int64_t os1, int M, int N, int K, float alpha, float beta, int sigmoid, int out_half,
                    hipStream_t st) {
-  const int64_t total = (int64_t)M * N;
-  if (total <= 0) return XFC_OK;
-  hipLaunchKernelGGL(generic_gemm_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st,
+  if (M <= 0 || N <= 0) return XFC_OK;
+  const int64_t tiles = (int64_t)ceil_div(M, GEN_T) * ceil_div(N, GEN_T);
+  if (tiles > 0x7fffffff) return XFC_ERR_INVALID;
+  hipLaunchKernelGGL(generic_gemm_kernel, dim3((unsigned)tiles), dim3(256), 0, st,
                      reinterpret_cast<const half_t*>(in1), as0, as1, reinterpret_cast<const half_t*>(in2), bs0, bs1,
                      out, os0, os1, M, N, K, alpha, beta, sigmoid, out_half);
   return check_launch();

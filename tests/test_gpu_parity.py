@@ -335,6 +335,19 @@ def test_xfc_gemm_any_stride_fallback_and_errors(dev):
     gi = torch.empty(B, d, device=dev)
     xfc_gemm(out, Wd, gi, 2.0, 0.0, False)
     assert rel(gi, O.dx(out.float().cpu(), W.float(), 2.0)) <= TOL
+    # several tiles of the fallback kernel with ragged edges on every axis and beta != 0, in the three layouts
+    M, N, K = 130, 201, 77
+    A, Bm = (torch.randn(M, K, generator=g) * 0.3).half(), (torch.randn(K, N, generator=g) * 0.3).half()
+    prev = torch.randn(M, N, generator=g)
+    want = 1.5 * (A.float() @ Bm.float()) - 0.5 * prev
+    for a_dev in (A.to(dev), A.t().contiguous().to(dev).t()):  # row x row, column x row
+        acc = prev.to(dev)
+        xfc_gemm(a_dev, Bm.to(dev), acc, 1.5, -0.5, False)
+        assert rel(acc, want) <= TOL and worst(acc, want) <= 2e-3 * float(want.abs().max())
+    acc = prev.half().to(dev)
+    xfc_gemm(A.to(dev), Bm.t().contiguous().to(dev).t(), acc, 1.5, -0.5, True)  # row x column, sigmoid
+    want = torch.sigmoid(1.5 * (A.float() @ Bm.float()) - 0.5 * prev.half().float())
+    assert rel(acc, want) <= TOL and worst(acc, want) <= 1e-3
     with pytest.raises(XfcError):  # row x row with apply_sigmoid: the reference exits the process here
         xfc_gemm(Xd, Wd.t().contiguous(), out, 1.0, 0.0, True)
     with pytest.raises(XfcError):  # inner dimensions disagree
