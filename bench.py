@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
 # HBM bytes per launch of the dW+update kernel: rocprofv3 --pmc FETCH_SIZE (KiB, x2.000 from the 1 GiB
 # copy in the same run) + WRITE_SIZE (KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
-DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2798712.4 + 1.000 * 3932160.0) * 1024.0,
+DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2799701.8 + 1.000 * 3932160.0) * 1024.0,
                            # the other configurations: profiles/xfc_step_other_configs_hbm_traffic_pmc.md
                            1: (2.000 * 285086.0 + 1.000 * 393216.0) * 1024.0,
                            3: (2.000 * 8560528.2 + 1.000 * 8436843.0) * 1024.0,
@@ -186,6 +186,28 @@ def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, wall_clock: b
         e1.record()
         torch.cuda.synchronize()
         out["copy_gbs"] = 2.0 * nbytes * n / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        # the same step with the update left unfused (the split-accumulation path: dW written as fp32, then a
+        # streaming SGD-momentum kernel over W, M and dW): what the fused epilogue is to be compared with, and what
+        # a pure read-modify-write stream of the update's shape reaches on this box
+        n = 5
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(n + 1)]
+        for i in range(n + 1):  # the first one allocates the gradient and is not counted
+            restore()
+            layer.fwd_grad(X, rowptr=rowptr, colidx=colidx)
+            layer.dx(B, scale=1.0)
+            ev[i][0].record()
+            layer.dw_accumulate(X)
+            ev[i][1].record()
+            layer.optimizer_step()
+            ev[i][2].record()
+        torch.cuda.synchronize()
+        dw_ms = sum(e[0].elapsed_time(e[1]) for e in ev[1:]) / n
+        upd_ms = sum(e[1].elapsed_time(e[2]) for e in ev[1:]) / n
+        out["unfused_update"] = {"dw_fp32_out_ms": dw_ms, "sgd_momentum_ms": upd_ms,
+                                 "sgd_momentum_gbs": 12.0 * L * d / (upd_ms * 1e-3) / 1e9,
+                                 "note": "xfc_dw (beta 0) + xfc_sgd_momentum in place of the fused dw_update; the "
+                                         "streaming kernel moves 12 bytes per weight (W and M read and written, "
+                                         "fp32 dW read)"}
     if loss_variant:
         # the forward pass of the reference's one step in a hundred: the same kernel with the summed BCE loss,
         # timed inside whole steps like the figure it is compared with (a forward pass run back to back with
@@ -359,6 +381,7 @@ def main() -> int:
         "step_tflops": wall_tf,
         "mfma_peak_frac": wall_tf / MFMA_F16_PEAK_TFLOPS,
         "copy_gbs": r.get("copy_gbs"),
+        "unfused_update": r.get("unfused_update"),
         "kernels_ms": s["kernels_ms"],
         "fwd_grad_with_loss_ms": r.get("fwd_grad_with_loss_ms"),
         "kernels_tflops": {"fwd_grad": gemm_flop / k_ms[0] / 1e9, "dx": gemm_flop / k_ms[1] / 1e9,
