@@ -472,10 +472,19 @@ def test_seeded_shape_sweep(dev):
         Xd = wide.to(dev)[:, :d]
         ref = O.step(X.float(), W.float(), torch.zeros(L, d), px, py, 0.05, 0.9, wd, scale)
         dX = lay.xfc_backward(Xd, px.to(dev), py.to(dev), scale=scale)
-        assert rel(lay.outsoft[:B, :L], ref["G"]) <= TOL
-        assert rel(dX[:B], ref["dX"]) <= TOL
-        assert rel(lay.xfc_weight, ref["W"]) <= TOL
-        assert rel(lay.momentum_buffer, ref["M"]) <= TOL
+        assert rel(lay.outsoft[:B, :L], ref["G"]) <= TOL and worst(lay.outsoft[:B, :L], ref["G"]) <= 2e-3
+        assert rel(dX[:B], ref["dX"]) <= TOL and worst(dX[:B], ref["dX"]) <= 5e-3
+        assert rel(lay.xfc_weight, ref["W"]) <= TOL and worst(lay.xfc_weight, ref["W"]) <= 3e-3
+        assert rel(lay.momentum_buffer, ref["M"]) <= TOL and worst(lay.momentum_buffer, ref["M"]) <= 3e-3
+
+
+@pytest.mark.parametrize("B,L,d", [(1030, 2500, 256), (2500, 1999, 128), (4100, 1024, 64)])
+def test_batches_above_1024(dev, B, L, d):
+    """More rows than any BASELINE configuration has: five to seventeen row tiles in the forward pass and dX, a
+    contraction over up to 4100 rows in dW."""
+    X, W, P = _problem(B, L, d, seed=B)
+    px, py = P.coo()
+    _check_step(dev, X, W, px, py, wd=1e-4, scale=2.0)
 
 
 def test_index_tensors_are_checked_and_moved_before_any_launch(dev):
