@@ -501,7 +501,7 @@ def test_index_tensors_are_checked_and_moved_before_any_launch(dev):
     assert torch.equal(G_dev, G_cpu)
     G_csr = lay.fwd_grad(Xd, rowptr=rp, colidx=ci).clone()        # CPU CSR
     assert torch.equal(G_dev, G_csr)
-    marker = lay.outsoft[:B].clone()
+    marker = lay.outsoft[:B, :L].clone()  # columns past the labels are never written (and may hold NaN)
     with pytest.raises(TypeError):
         lay.fwd_grad(Xd, rowptr=rp.long(), colidx=ci)             # int64 CSR is not silently misread
     with pytest.raises(TypeError):
@@ -516,7 +516,7 @@ def test_index_tensors_are_checked_and_moved_before_any_launch(dev):
     with pytest.raises(ValueError):
         small.fwd_grad(Xd, px, py)
     torch.cuda.synchronize()
-    assert torch.equal(lay.outsoft[:B], marker)                   # nothing ran for the rejected calls
+    assert torch.equal(lay.outsoft[:B, :L], marker)                   # nothing ran for the rejected calls
     gi = lay.step_csr(Xd, rp, ci)                                 # CPU CSR through the one-call step
     ref = O.step(X.float(), W.float(), torch.zeros(L, d), px, py, 0.05, 0.9, 0.0, 1.0)
     assert rel(gi, ref["dX"]) <= TOL and rel(lay.xfc_weight, ref["W"]) <= TOL
