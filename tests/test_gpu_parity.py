@@ -487,6 +487,16 @@ def test_batches_above_1024(dev, B, L, d):
     _check_step(dev, X, W, px, py, wd=1e-4, scale=2.0)
 
 
+@pytest.mark.parametrize("B,L,d,csr", [(16, 3_200_000, 8, False), (16, 3_200_000, 8, True), (15000, 520, 8, True)])
+def test_bucket_pass_variants(dev, B, L, d, csr):
+    """The pass that groups the positives by label tile keeps its per-tile counters in LDS up to 12,288 label tiles
+    and in global memory above (3.2 M labels: 12,500 tiles), and walks a CSR list by entry with the row pointers in
+    LDS while they fit next to the counters (15,000 rows do not: one row per thread then)."""
+    X, W, P = _problem(B, L, d, kmax=6, kmean=3.0, seed=77)
+    px, py = P.coo()
+    _check_step(dev, X, W, px, py, csr=(torch.from_numpy(P.rowptr), torch.from_numpy(P.colidx)) if csr else None)
+
+
 def test_index_tensors_are_checked_and_moved_before_any_launch(dev):
     """Label tensors arrive from the collator on the CPU (dl_base.py:934-936).  They are copied to the
     layer's GPU, never dereferenced where they are; a wrong dtype or length raises before a launch."""
