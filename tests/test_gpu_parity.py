@@ -117,6 +117,16 @@ def test_adversarial_label_sets(dev):
     G2 = lay.fwd_grad(X.to(dev), px2.to(dev), py2.to(dev)).clone()
     G1 = lay.fwd_grad(X.to(dev), px.to(dev), py.to(dev))
     assert torch.equal(G1, G2)
+    # row pointers that are not a CSR (not monotone, negative, past the list): nothing outside colidx[0 .. nnz) is
+    # read and no entry counts twice, so at most nnz entries of G are below zero and the rest is sigmoid(Z)
+    rp, ci = coo_to_csr(px, py, B)
+    bad = rp.clone()
+    bad[1:-1] = torch.from_numpy(np.random.default_rng(1).integers(-5, len(ci) + 50, size=B - 1).astype(np.int32))
+    Gb = lay.fwd_grad(X.to(dev), rowptr=bad.to(dev), colidx=ci.to(dev)).float().cpu()
+    S = torch.sigmoid(O.logits(X.float(), W.float()))
+    neg = Gb < 0
+    assert int(neg.sum()) <= len(ci) and rel(Gb[~neg], S[~neg]) <= TOL
+    assert float((Gb[neg] - (S[neg] - 1.0)).abs().max()) <= 1e-3
     # no positives at all: G = sigmoid(Z)
     G0 = lay.fwd_grad(X.to(dev))
     assert rel(G0, torch.sigmoid(O.logits(X.float(), W.float()))) <= TOL
