@@ -88,7 +88,10 @@ int xfc_logits(const void* X, int64_t ldx, const void* W, int64_t ldw, void* out
  * reference's non-accumulating indexed update does; pairs outside [0,B)x[0,L)
  * are ignored.  Positives come either as CSR (rowptr int32[B+1], colidx
  * int32[nnz]) or as the reference's COO pair (pos_x, pos_y int64[nnz],
- * dl_base.py:934-936), in any order.
+ * dl_base.py:934-936), in any order.  Of colidx the device code reads
+ * colidx[max(rowptr[0],0) .. min(rowptr[B],nnz)) and nothing else, each entry
+ * once, whatever rowptr holds; row pointers that do not ascend give an
+ * unspecified subset of those entries to unspecified rows.
  * G has leading dimension ldg >= L, a multiple of 8; the columns
  * L .. round_up(L,8)-1 are written as zero (xfc_dx / xfc_dw_update rely on it).
  * If `loss` is non-NULL it receives the summed BCE-with-logits loss of the batch,
