@@ -642,6 +642,46 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
     }
   };
   auto for_each = [&](auto&& f) { for_each_block(1, f); };
+  // f(key, index) for every element of the row whose key is at least kthr.  Almost none is, so two elements at a
+  // time are first tested in packed 16-bit arithmetic: flipping the magnitude bits of a negative fp16 pattern gives
+  // a signed 16-bit integer x = key - 32768 (except that -0 gives -1 where its key is that of +0, hence the
+  // threshold one lower), and min(x, t - 1) != x exactly when x >= t.  Only a 16-byte piece with a hit goes through
+  // the exact per-element test.  Two pieces per thread are in flight.
+  auto for_each_from = [&](uint32_t kthr, auto&& f) {
+    typedef short short2v __attribute__((ext_vector_type(2)));
+    const int xq = (int)kthr - 32768 - 1;  // quick test: x >= xq
+    const bool all = xq <= -32768;
+    const uint32_t t2 = ((uint32_t)(xq - 1) & 0xffffu) * 0x10001u;
+    const short2v tv = __builtin_bit_cast(short2v, t2);
+    auto piece = [&](const uint4v& q, int i) {
+      uint32_t changed = 0u;
+#pragma unroll
+      for (int e2 = 0; e2 < 4; ++e2) {
+        const uint32_t pair = q[e2];  // (a bit cast straight from the element expression reads element 0)
+        const short2v h = __builtin_bit_cast(short2v, pair);
+        const short2v x = h ^ ((h >> (short2v)(15)) & (short2v)(0x7fff));
+        const short2v m = __builtin_elementwise_min(x, tv);
+        changed |= __builtin_bit_cast(uint32_t, m) ^ __builtin_bit_cast(uint32_t, x);
+      }
+      if (all || changed != 0u) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t key = sel_key((q[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+          if (i + e < L && key >= kthr) f(key, i + e);
+        }
+      }
+    };
+    constexpr int64_t STEP = (int64_t)SEL_THREADS * 8;
+    for (int64_t i64 = tid * 8; i64 < L; i64 += 2 * STEP) {
+      const int i = (int)i64;
+      const bool second = i64 + STEP < L;
+      const uint4v q0 = *reinterpret_cast<const uint4v*>(row + i);
+      uint4v q1 = {0u, 0u, 0u, 0u};
+      if (second) q1 = *reinterpret_cast<const uint4v*>(row + i + STEP);
+      piece(q0, i);
+      if (second) piece(q1, i + (int)STEP);
+    }
+  };
   auto push = [&](uint32_t key, int idx) {
     const int slot = atomicAdd(&S.n_cand, 1);
     if (slot < SEL_CAP) S.cand[slot] = ((unsigned long long)(0xffffu - key) << 32) | (uint32_t)idx;
@@ -683,7 +723,7 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
     find_bin(SEL_BINS, 0);  // the host only asks for a sample that holds at least K elements
     __syncthreads();
     const int sbin = S.bin;
-    for_each([&](uint32_t key, int idx) { if ((int)(key >> 5) >= sbin) push(key, idx); });
+    for_each_from((uint32_t)sbin << 5, [&](uint32_t key, int idx) { push(key, idx); });
     __syncthreads();
     done = S.n_cand <= SEL_CAP;  // counts every push, also those that found the buffer full
     __syncthreads();
@@ -707,7 +747,7 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
   if (done) {
     // the sampled bound already gathered a superset of the answer
   } else if (above + in_bin <= SEL_CAP) {
-    for_each([&](uint32_t key, int idx) { if ((int)(key >> 5) >= bin) push(key, idx); });
+    for_each_from((uint32_t)bin << 5, [&](uint32_t key, int idx) { push(key, idx); });
   } else {
     if (tid < 64) S.hist[tid] = 0;
     __syncthreads();
@@ -719,10 +759,10 @@ __global__ void __launch_bounds__(SEL_THREADS) topk_select_kernel(const half_t* 
     const int n_gt = S.above, n_eq = S.hist[S.bin];
     __syncthreads();
     if (n_gt + n_eq <= SEL_CAP) {
-      for_each([&](uint32_t key, int idx) { if (key >= thr) push(key, idx); });
+      for_each_from(thr, [&](uint32_t key, int idx) { push(key, idx); });
     } else {
       // too many copies of the K-th value to sort: those above it first, then its copies in label order
-      for_each([&](uint32_t key, int idx) { if (key > thr) push(key, idx); });
+      for_each_from(thr + 1u, [&](uint32_t key, int idx) { push(key, idx); });
       const int need = K - n_gt;
       int taken = 0;
       for (int base = 0; base < L && taken < need; base += SEL_THREADS * 8) {
