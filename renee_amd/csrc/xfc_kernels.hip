@@ -978,18 +978,24 @@ __global__ void __launch_bounds__(DwCore::NT) dw_kernel(DwArgs a) {
     constexpr int DEPTH = MODE == DW_UPDATE_MASTER ? 2 : 4;  // the fp32 pieces take twice the registers per strip (2-6 measure alike)
     auto strip_row = [&](int s) { return m0 + wm * C::TM + (s / (4 * (C::FN / 2))) * 32 + 8 * ((s / (C::FN / 2)) % 4) + srow; };
     auto strip_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 8; };
+    // The fp32 arrays (dW out, master W and M) are touched in two 16-byte pieces per lane and strip.  With a lane
+    // on 8 consecutive dims each piece's instruction would write every other 16 bytes of a line; there a lane
+    // takes dims c .. c+3 and c+32 .. c+35 instead, so that eight lanes cover a whole 128-byte line each time.
+    constexpr bool SPLIT = MODE != DW_UPDATE;
+    auto split_col = [&](int s) { return n0 + wn * C::TN + (s % (C::FN / 2)) * 64 + sch * 4; };
     half8 wq[DEPTH], mq[DEPTH];
     float4v w32q[DEPTH][2], m32q[DEPTH][2];  // DW_UPDATE_MASTER
     auto fetch32 = [&](int s, float4v (&wv)[2], float4v (&mv)[2]) {
-      int row = strip_row(s), col = strip_col(s);
+      int row = strip_row(s), c0 = split_col(s), c1 = c0 + 32;
       row = row < a.M ? row : a.M - 1;
-      col = col < a.N ? col : a.N - 8;
-      const float* wp = a.W32 + (int64_t)row * a.ldw32 + col;
-      const float* mp = a.M32 + (int64_t)row * a.ldm32 + col;
-      wv[0] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(wp));
-      wv[1] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(wp + 4));
-      mv[0] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(mp));
-      mv[1] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(mp + 4));
+      c0 = c0 < a.N ? c0 : a.N - 4;
+      c1 = c1 < a.N ? c1 : a.N - 4;
+      const float* wp = a.W32 + (int64_t)row * a.ldw32;
+      const float* mp = a.M32 + (int64_t)row * a.ldm32;
+      wv[0] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(wp + c0));
+      wv[1] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(wp + c1));
+      mv[0] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(mp + c0));
+      mv[1] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(mp + c1));
     };
     // unconditional (out-of-range strips read the last valid row / column block and are not stored):
     // straight-line loads let the compiler count exactly how many may stay in flight at each use
@@ -1018,35 +1024,37 @@ __global__ void __launch_bounds__(DwCore::NT) dw_kernel(DwArgs a) {
           stage[(4 * h + rr) * 64 + f * 32 + (lane & 31)] = acc[fm][2 * fp + f][4 * q + rr];
       // the wave's own LDS traffic is ordered: the writes above are visible to the reads below
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      const float4v v0 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8);
-      const float4v v1 = *reinterpret_cast<const float4v*>(stage + srow * 64 + sch * 8 + 4);
+      const float4v v0 = *reinterpret_cast<const float4v*>(stage + srow * 64 + (SPLIT ? sch * 4 : sch * 8));
+      const float4v v1 = *reinterpret_cast<const float4v*>(stage + srow * 64 + (SPLIT ? 32 + sch * 4 : sch * 8 + 4));
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const int row = strip_row(s), col = strip_col(s);
-      const bool in = row < a.M && col < a.N;
+      const int row = strip_row(s), col = SPLIT ? split_col(s) : strip_col(s);
+      const int col1 = SPLIT ? col + 32 : col + 4;  // first dim of the lane's second piece
+      const bool in = row < a.M && col < a.N, in1 = row < a.M && col1 < a.N;
       const float g[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
       if constexpr (MODE == DW_OUT) {
-        if (in) {
-          float* o = a.out + (int64_t)row * a.ldo + col;
-          float4v o0, o1;
+        float* orow = a.out + (int64_t)row * a.ldo;
+        float4v o0, o1;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
-          if (a.beta != 0.f) {
-            o0 += a.beta * *reinterpret_cast<const float4v*>(o);
-            o1 += a.beta * *reinterpret_cast<const float4v*>(o + 4);
-          }
-          *reinterpret_cast<float4v*>(o) = o0;
-          *reinterpret_cast<float4v*>(o + 4) = o1;
+        for (int e = 0; e < 4; ++e) { o0[e] = a.alpha * g[e]; o1[e] = a.alpha * g[4 + e]; }
+        if (a.beta != 0.f) {  // both pieces' loads before either store
+          float4v p0 = {0.f, 0.f, 0.f, 0.f}, p1 = {0.f, 0.f, 0.f, 0.f};
+          if (in) p0 = *reinterpret_cast<const float4v*>(orow + col);
+          if (in1) p1 = *reinterpret_cast<const float4v*>(orow + col1);
+          o0 += a.beta * p0;
+          o1 += a.beta * p1;
         }
+        if (in) *reinterpret_cast<float4v*>(orow + col) = o0;
+        if (in1) *reinterpret_cast<float4v*>(orow + col1) = o1;
       } else if constexpr (MODE == DW_UPDATE_MASTER) {
         // the reference's regime (fp32 parameter and FusedSGD state, dl_base.py:185, main.py:178-179) with the
         // per-step fp16 cast of W (dl_base.py:562) written from the same pass
         float4v wv[2] = {w32q[s % DEPTH][0], w32q[s % DEPTH][1]}, mv[2] = {m32q[s % DEPTH][0], m32q[s % DEPTH][1]};
         if (s + DEPTH < NS) fetch32(s + DEPTH, w32q[s % DEPTH], m32q[s % DEPTH]);
-        if (in) {
+        if (in) {  // the second piece lies 32 dims past the first: when it is inside N, so is the first
           if (a.dw_dump) {
-            float* d = a.dw_dump + (int64_t)row * a.ld_dump + col;
-            *reinterpret_cast<float4v*>(d) = v0;
-            *reinterpret_cast<float4v*>(d + 4) = v1;
+            float* d = a.dw_dump + (int64_t)row * a.ld_dump;
+            *reinterpret_cast<float4v*>(d + col) = v0;
+            if (in1) *reinterpret_cast<float4v*>(d + col1) = v1;
           }
           half8 w16;
 #pragma unroll
@@ -1063,13 +1071,18 @@ __global__ void __launch_bounds__(DwCore::NT) dw_kernel(DwArgs a) {
             wv[e >> 2][e & 3] = wn;
             w16[e] = (half_t)wn;
           }
-          float* wp = a.W32 + (int64_t)row * a.ldw32 + col;
-          float* mp = a.M32 + (int64_t)row * a.ldm32 + col;
-          *reinterpret_cast<float4v*>(mp) = mv[0];
-          *reinterpret_cast<float4v*>(mp + 4) = mv[1];
-          *reinterpret_cast<float4v*>(wp) = wv[0];
-          *reinterpret_cast<float4v*>(wp + 4) = wv[1];
-          *reinterpret_cast<half8*>(a.Wt + (int64_t)row * a.ldw + col) = w16;
+          typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+          float* wp = a.W32 + (int64_t)row * a.ldw32;
+          float* mp = a.M32 + (int64_t)row * a.ldm32;
+          half_t* hp = a.Wt + (int64_t)row * a.ldw;
+          *reinterpret_cast<float4v*>(mp + col) = mv[0];
+          *reinterpret_cast<float4v*>(wp + col) = wv[0];
+          *reinterpret_cast<half4*>(hp + col) = half4{w16[0], w16[1], w16[2], w16[3]};
+          if (in1) {
+            *reinterpret_cast<float4v*>(mp + col1) = mv[1];
+            *reinterpret_cast<float4v*>(wp + col1) = wv[1];
+            *reinterpret_cast<half4*>(hp + col1) = half4{w16[4], w16[5], w16[6], w16[7]};
+          }
         }
       } else {
         half8 wv = wq[s % DEPTH], mv = mq[s % DEPTH];
