@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, AMD's published figure
 
 # HBM bytes per launch of the dW+update kernel: rocprofv3 --pmc FETCH_SIZE (KiB, x2.000 from the 1 GiB
 # copy in the same run) + WRITE_SIZE (KiB, x1.000); see profiles/xfc_step_cfg2_hbm_traffic_pmc.md.
-DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2799701.8 + 1.000 * 3932160.0) * 1024.0,
+DW_UPDATE_TRAFFIC_BYTES = {2: (2.000 * 2800162.7 + 1.000 * 3932160.0) * 1024.0,
                            # the other configurations: profiles/xfc_step_other_configs_hbm_traffic_pmc.md
                            1: (2.000 * 285086.0 + 1.000 * 393216.0) * 1024.0,
                            3: (2.000 * 8560528.2 + 1.000 * 8436843.0) * 1024.0,
