@@ -107,7 +107,7 @@ def cpu_baseline_cfg0(d: int, seed: int):
 
 
 def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, wall_clock: bool = True, scorers: bool = False,
-                batch: int = 0, loss_variant: bool = False):
+                batch: int = 0, loss_variant: bool = False, graph: bool = False):
     """Times `steps` steps of one BASELINE configuration (with `batch` rows instead of its own when
     given), each from the same (W0, M1) state."""
     import torch
@@ -224,6 +224,30 @@ def time_config(cfg: int, steps: int, warmup: int, seed: int, dev, wall_clock: b
             layer.dw_update(X)
         torch.cuda.synchronize()
         out["fwd_grad_with_loss_ms"] = sum(e[0].elapsed_time(e[1]) for e in ev[1:]) / n
+    if graph:
+        # The same step captured once as a HIP graph (xfc_step_csr: the entry points enqueue on the caller's stream
+        # and neither allocate nor synchronise) and replayed back to back: what a small batch costs when the host's
+        # launch gaps between the five kernels are taken out.
+        restore()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                layer.step_csr(X, rowptr, colidx)
+        torch.cuda.current_stream().wait_stream(side)
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        out["graph_replay_ms_per_step"] = e0.elapsed_time(e1) / steps
+        del g
     if scorers:
         restore()
         for K in (5, 100):
@@ -319,7 +343,7 @@ def summarise(r, cfg=None):
     if cfg in DW_UPDATE_TRAFFIC_BYTES:
         s["dw_update_traffic"] = DW_UPDATE_TRAFFIC_BYTES[cfg]
         s["dw_update_gbs_incl_measured_traffic"] = DW_UPDATE_TRAFFIC_BYTES[cfg] / (r["k_ms"][2] * 1e-3) / 1e9
-    for k in ("wall_ms_per_step", "ms_events", "copy_gbs", "top5_ms", "top100_ms"):
+    for k in ("wall_ms_per_step", "ms_events", "copy_gbs", "top5_ms", "top100_ms", "graph_replay_ms_per_step"):
         if k in r:
             s[k] = r[k]
     if "top5_ms" in r:
@@ -416,7 +440,7 @@ def main() -> int:
             if cfg == args.config:
                 continue
             others[f"configs[{cfg}]"] = summarise(time_config(cfg, n, 2, args.seed, dev, wall_clock=False,
-                                                              scorers=(cfg == 3)), cfg)
+                                                              scorers=(cfg == 3), graph=(cfg in (0, 1))), cfg)
             others[f"configs[{cfg}]"]["steps"] = n
         # what the 64-row tiles buy at batch 32: the same label count at batch 256 (one full-height tile)
         b256 = time_config(0, 20, 2, args.seed, dev, wall_clock=False, batch=256)["ms_per_step"]
