@@ -7,7 +7,7 @@ reference's kind of schedule (lr1 = 0.0025, cosine with warm-up from 0, dl_base.
 arithmetic is the oracle's fp32 update; the fp16-resident regime rounds W and M to fp16 after each step
 (what xfc_dw_update stores), the master regime rounds only the copy the GEMMs read.  It records how many
 updates the fp16 store drops (|lr * M| below half an ulp of W) and bounds the drift of the trained
-weights; the numbers are quoted in DESIGN.md."""
+weights."""
 import math
 
 import pytest
